@@ -61,7 +61,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const int* __restrict__ token_request, const int* __restrict__ positions, T* __restrict__ out,
     int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
     int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits,
-    const float* __restrict__ slopes, int v_dim, int64_t v_row_stride, int has_sink, float sink_logit) {
+    const float* __restrict__ slopes, int v_dim, int64_t v_row_stride, int has_sink, float sink_logit, int mask_chunk) {
   using S = typename SumType<T>::type;
   extern __shared__ __align__(8) unsigned char q_lds_bytes[];
   S* q_lds = reinterpret_cast<S*>(q_lds_bytes);  // [GT][head_dim], pre-multiplied by the scale
@@ -84,7 +84,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 
   const int pos = positions[t];
   const int req = token_request[t];
-  const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
+  // (a chunked mask: only the keys of the query's own stretch of `mask_chunk` positions, counted from 0)
+  const int lo = max((window > 0) ? max(0, pos - window + 1) : 0, (mask_chunk > 0) ? pos / mask_chunk * mask_chunk : 0);
   const int hi = pos + 1;
   int chunk = (hi - lo + num_splits - 1) / num_splits;
   chunk = (chunk + MI_WAVE - 1) / MI_WAVE * MI_WAVE;
@@ -331,7 +332,7 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
                                int num_tokens, int q_heads, int kv_heads, int head_dim,
                                int page_size, float scale, int window, int num_splits,
                                const float* slopes, hipStream_t stream, int v_dim = 0, int64_t v_row_stride = 0,
-                               int has_sink = 0, float sink_logit = 0.f) {
+                               int has_sink = 0, float sink_logit = 0.f, int mask_chunk = 0) {
   // (values as wide as the keys and packed, no sink: what the callers that say nothing mean)
   if (v_dim <= 0) v_dim = head_dim;
   if (v_row_stride <= 0) v_row_stride = v_dim;
@@ -343,7 +344,7 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
   attn_generic_kernel<T, VPL, VEC><<<grid, MI_WAVE, lds, stream>>>(                               \
       (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
       token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
-      head_dim, page_size, scale, window, num_splits, slopes, v_dim, v_row_stride, has_sink, sink_logit)
+      head_dim, page_size, scale, window, num_splits, slopes, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk)
   if (v_dim <= 64) { if (vec) MI_ATTN_LAUNCH(1, true); else MI_ATTN_LAUNCH(1, false); }
   else if (v_dim <= 128) { if (vec) MI_ATTN_LAUNCH(2, true); else MI_ATTN_LAUNCH(2, false); }
   else if (v_dim <= 256) { if (vec) MI_ATTN_LAUNCH(4, true); else MI_ATTN_LAUNCH(4, false); }
@@ -413,7 +414,8 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
 // elements that lie `v_row_stride` elements apart (a value row may be the front part of a key
 // row: pass the key pages as value pages and head_dim as the stride), key rows up to 1024 wide,
 // and optionally a sink: one more term exp(sink_logit) in the softmax's denominator that
-// carries no value.  Queries are [token][head][head_dim], outputs [token][head][v_dim];
+// carries no value, and optionally a chunked mask: a query sees only the keys of its own
+// stretch of `mask_chunk` positions (0: none).  Queries are [token][head][head_dim], outputs [token][head][v_dim];
 // part_acc holds num_tokens*q_heads*num_splits*v_dim floats.
 extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
                                const void* v_pages, const int* block_table, int max_blocks,
@@ -422,7 +424,8 @@ extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, c
                                int num_tokens, int q_heads, int kv_heads, int head_dim, int v_dim,
                                int64_t v_row_stride, int page_size, int num_pages, float scale, int window,
                                int num_splits, const float* slopes, int has_sink, float sink_logit,
-                               hipStream_t stream) {
+                               int mask_chunk, hipStream_t stream) {
+  MI_REQUIRE(mask_chunk >= 0, "attn_general: mask_chunk=%d must be 0 (none) or positive", mask_chunk);
   MI_REQUIRE(v_dim > 0 && v_row_stride >= v_dim, "attn_general: value rows of %d lie %lld apart", v_dim,
              (long long)v_row_stride);
   const int bad = attn_generic_check(dtype, q_row_stride, max_blocks, out_row_stride, num_tokens, q_heads,
@@ -434,11 +437,11 @@ extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, c
     return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                       token_request, positions, out, out_row_stride, part_acc, part_ml,
                                       num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                      num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit);
+                                      num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk);
   return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                     num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit);
+                                     num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk);
 }
 
 // The combining step alone, for partials written by the matrix-core kernel.

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
     int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request,
-    int pair_group, int first_token, int has_sink, float sink_log2) {
+    int pair_group, int first_token, int has_sink, float sink_log2, int mask_chunk) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   // PS != 0: the page size is this constant (divisions become shifts, value offsets
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     token[rg] = t0 + tok_in_tile;
     head[rg] = kvh * group + g0 + head_in_block;
     pos[rg] = pos0 + tok_in_tile;
-    lo_row[rg] = (window > 0) ? max(0, pos[rg] - window + 1) : 0;
+    lo_row[rg] = max((window > 0) ? max(0, pos[rg] - window + 1) : 0, (mask_chunk > 0) ? pos[rg] / mask_chunk * mask_chunk : 0);
   }
 
   // smallest position and largest window start among this wave's rows (for the mask-free test)
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   wave_lo_max = __builtin_amdgcn_readfirstlane(wave_lo_max);
 
   // ---- key range of this block ------------------------------------------------
-  const int tile_lo = (window > 0) ? max(0, pos0 - window + 1) : 0;
+  const int tile_lo = max((window > 0) ? max(0, pos0 - window + 1) : 0, (mask_chunk > 0) ? pos0 / mask_chunk * mask_chunk : 0);
   const int tile_hi = pos0 + n_tok;  // exclusive
   int chunk = (tile_hi - tile_lo + num_splits - 1) / num_splits;
   chunk = (chunk + 31) / 32 * 32;
@@ -809,7 +809,9 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             float* part_acc, float* part_ml, int q_heads, int kv_heads,
                             int head_dim, int page_size, int num_pages, float scale, int window,
                             int num_splits, int shape, int one_tile_per_request,
-                            int first_token, int combine, int has_sink, float sink_logit, hipStream_t stream) {
+                            int first_token, int combine, int has_sink, float sink_logit, int mask_chunk,
+                            hipStream_t stream) {
+  MI_REQUIRE(mask_chunk >= 0, "attn_mfma: mask_chunk=%d must be 0 (none) or positive", mask_chunk);
   MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
              "attn_mfma: bad sizes tokens=%d requests=%d tiles=%d", num_tokens, num_requests, num_tiles);
@@ -868,7 +870,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
-      num_splits, hb, tq, one_tile_per_request, pair_group, first_token, has_sink, sink_logit * LOG2E)
+      num_splits, hb, tq, one_tile_per_request, pair_group, first_token, has_sink, sink_logit * LOG2E, mask_chunk)
 // (head sizes above 128 have no wide shape and were refused above: their cases name the 128 kernel,
 // so that nothing is compiled for them)
 #define MI_LAUNCH_P(DD, PP)                                                                       \

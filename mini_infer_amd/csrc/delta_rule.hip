@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const T* __restrict__ tail,
     int64_t tail_stride, const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ token_request, T* __restrict__ y, int64_t y_stride, int channels, int taps,
-    int num_slots, int row0) {
+    int num_slots, int row0, const float* __restrict__ bias) {
   const int t = row0 + blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
@@ -45,8 +45,9 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
   const T* mine = tail + (int64_t)((slot < 0 || slot >= num_slots) ? num_slots : slot) * tail_stride;
   const float* wc = w + (int64_t)c * taps;
   const int back = taps - 1;
+  const float start = bias ? bias[c] : 0.f;  // (a convolution with a bias per channel starts its sum there)
   if constexpr (sizeof(T) == 4) {
-    double sum = 0.0;
+    double sum = (double)start;
     for (int j = 0; j < taps; ++j) {
       const int at = i - back + j;  // row of the portion, negative: of the tail
       const float v = at >= 0 ? x[(int64_t)(t - back + j) * x_stride + c] : mine[(int64_t)(back + at) * channels + c];
@@ -54,7 +55,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
     }
     y[(int64_t)t * y_stride + c] = (float)(sum / (1.0 + exp(-sum)));
   } else {
-    float sum = 0.f;
+    float sum = start;
     for (int j = 0; j < taps; ++j) {
       const int at = i - back + j;
       const float v = at >= 0 ? to_f32(x[(int64_t)(t - back + j) * x_stride + c])
@@ -93,12 +94,13 @@ template <typename T>
 __global__ __launch_bounds__(256) void short_conv_walk_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, T* __restrict__ tail, int64_t tail_stride,
     const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ y, int64_t y_stride, int channels, int taps,
-    int num_slots) {
+    int num_slots, const float* __restrict__ bias) {
   const int b = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
   const int first = cu[b], last = cu[b + 1];
   if (last <= first) return;
+  const float start = bias ? bias[c] : 0.f;
   const int slot = slots[b];
   T* mine = tail + (int64_t)((slot < 0 || slot >= num_slots) ? num_slots : slot) * tail_stride;
   const int back = taps - 1;
@@ -111,14 +113,14 @@ __global__ __launch_bounds__(256) void short_conv_walk_kernel(
   for (int t = first; t < last; ++t) {
     const float now = to_f32(x[(int64_t)t * x_stride + c]);
     if constexpr (sizeof(T) == 4) {
-      double sum = 0.0;
+      double sum = (double)start;
 #pragma unroll
       for (int j = 0; j < DELTA_MAX_TAPS; ++j)
         if (j < back) sum = fma((double)wc[j], (double)window[j], sum);
       sum = fma((double)w[(int64_t)c * taps + back], (double)now, sum);
       y[(int64_t)t * y_stride + c] = (float)(sum / (1.0 + exp(-sum)));
     } else {
-      float sum = 0.f;
+      float sum = start;
 #pragma unroll
       for (int j = 0; j < DELTA_MAX_TAPS; ++j)
         if (j < back) sum = fmaf(wc[j], window[j], sum);
@@ -413,11 +415,12 @@ static void delta_layout(int dim, int vdim, int* lanes, int* rows) {
 }  // namespace
 
 // x: the projections [tokens, >= channels] (row stride); w float32 [channels, taps]; tail
-// [slots + 1, (taps-1) * channels] in the element type (row stride); y [tokens, channels].
+// [slots + 1, (taps-1) * channels] in the element type (row stride); y [tokens, channels]; bias float32
+// [channels] or null.
 extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const float* w, void* tail,
                              int64_t tail_stride, const int* cu, const int* slots, const int* token_request,
                              void* y, int64_t y_stride, int num_tokens, int num_requests, int channels, int taps,
-                             int num_slots, hipStream_t stream) {
+                             int num_slots, const float* bias, hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && channels > 0, "short_conv: bad sizes tokens=%d requests=%d channels=%d",
              num_tokens, num_requests, channels);
   MI_REQUIRE(taps >= 1 && taps <= DELTA_MAX_TAPS, "short_conv: taps=%d must be 1..%d", taps, DELTA_MAX_TAPS);
@@ -432,10 +435,10 @@ extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const f
     dim3 grid(blocks, num_requests);
     if (dtype == MI_F32)
       short_conv_walk_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, w, (float*)tail, tail_stride, cu, slots,
-                                                              (float*)y, y_stride, channels, taps, num_slots);
+                                                              (float*)y, y_stride, channels, taps, num_slots, bias);
     else
       short_conv_walk_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_stride, w, (bf16_t*)tail, tail_stride, cu,
-                                                               slots, (bf16_t*)y, y_stride, channels, taps, num_slots);
+                                                               slots, (bf16_t*)y, y_stride, channels, taps, num_slots, bias);
     MI_CHECK_LAUNCH("short_conv_walk");
     return MI_OK;
   }
@@ -444,11 +447,11 @@ extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const f
     if (dtype == MI_F32)
       short_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, w, (const float*)tail, tail_stride, cu,
                                                          slots, token_request, (float*)y, y_stride, channels, taps,
-                                                         num_slots, first);
+                                                         num_slots, first, bias);
     else
       short_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_stride, w, (const bf16_t*)tail, tail_stride,
                                                           cu, slots, token_request, (bf16_t*)y, y_stride, channels, taps,
-                                                          num_slots, first);
+                                                          num_slots, first, bias);
   }
   MI_CHECK_LAUNCH("short_conv");
   if (taps > 1) {

@@ -24,6 +24,7 @@ from mini_infer_amd.engine.decode_graph import DecodeGraphs
 from mini_infer_amd.models import architecture_for
 from mini_infer_amd.parts.base import StepContext
 from mini_infer_amd.weights import load_checkpoint
+from mini_infer_amd.weights.safetensors_io import CheckpointReader
 from mini_infer_amd.weights.random_init import fill_random_on_device
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -119,6 +120,8 @@ class ModelRunner:
         raw = read_config_json(model_name)
         arch = architecture_for(raw)
         config = arch.parse_config(raw)
+        if arch.with_checkpoint_shapes is not None:
+            config = arch.with_checkpoint_shapes(config, CheckpointReader(model_name).shapes)
         model = arch.make_model(config, resolve_dtype(engine.dtype), dev)
         load_checkpoint(model, model_name)
         runner = cls(model, config, num_blocks=engine.num_blocks, block_size=engine.block_size,

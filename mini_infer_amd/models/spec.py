@@ -113,6 +113,9 @@ class Architecture:
     parse_config: Callable[[dict[str, Any]], Any]  # raw config.json keys -> typed config
     build_spec: Callable[[Any], ModelSpec] | None = None  # typed config -> ModelSpec
     build_model: Callable[[Any, Any, Any], Any] | None = None  # (typed config, dtype, device) -> model
+    # (typed config, {tensor name: shape} of the checkpoint) -> typed config: for designs in which a
+    # size is given by a tensor's shape and not by config.json; asked before the model is built
+    with_checkpoint_shapes: Callable[[Any, dict], Any] | None = None
 
     def __post_init__(self) -> None:
         if (self.build_spec is None) == (self.build_model is None):

@@ -911,6 +911,7 @@ def paged_attention(
     slopes: torch.Tensor | None = None,
     v_head_dim: int | None = None,
     sink_logit: float | None = None,
+    chunk: int | None = None,
 ) -> torch.Tensor | AttentionPieces:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
 
@@ -919,6 +920,10 @@ def paged_attention(
     of its key row.  `sink_logit`: the softmax's denominator gets one more term
     exp(sink_logit), a sink that carries no value (both attention kernels know it; uncombined
     `AttentionPieces` do not).  Values of a width of their own run the plain kernel.
+
+    `chunk`: a chunked mask: the token at position p sees only keys from `p // chunk * chunk` on
+    (its own stretch of `chunk` positions, counted from the sequence's start); it combines with
+    the causal order and with a window.  Uncombined `AttentionPieces` are not made with it.
 
     `slopes` (float32 [q_heads], optional): the score of head h for the key at position j
     seen from position p gets `slopes[h] * (j - p)` added before the softmax.  Only the
@@ -938,11 +943,16 @@ def paged_attention(
     bfloat16 caches with transposed values run on the matrix cores; everything else
     (float32, other head or page sizes) runs the plain kernel.
     """
-    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or (sink_logit is not None and not v_transposed):
+    if chunk is not None and chunk <= 0:
+        raise KernelShapeError(f"a chunked mask needs a positive chunk, got {chunk}")
+    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or (
+        (sink_logit is not None or chunk is not None) and not v_transposed
+    ):
         return _paged_attention_general(
             q, k_pages, v_pages, block_table, token_request, positions, q_heads=q_heads, kv_heads=kv_heads,
             head_dim=head_dim, v_head_dim=head_dim if v_head_dim is None else int(v_head_dim), scale=scale,
             window=window, max_seq_len=max_seq_len, v_transposed=v_transposed, slopes=slopes, sink_logit=sink_logit,
+            chunk=chunk,
         )
     _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, cu_seqlens_q)
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
@@ -1017,7 +1027,8 @@ def paged_attention(
                 _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
                 _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens, num_tiles, _ptr(out), out.stride(0),
                 _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads, head_dim, page_size, num_pages, float(scale),
-                int(window or 0), splits, shape, 0, 0, 1, int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
+                int(window or 0), splits, shape, 0, 0, 1, int(sink_logit is not None), float(sink_logit or 0.0),
+                int(chunk or 0), _stream(),
             )
         )
         return out
@@ -1060,7 +1071,8 @@ def paged_attention(
                     num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
                     shape, int(one_tile_per_request), first_token,
-                    0 if (leave_pieces and splits > 1) else 1, int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
+                    0 if (leave_pieces and splits > 1) else 1, int(sink_logit is not None), float(sink_logit or 0.0),
+                    int(chunk or 0), _stream(),
                 )
             )
             if leave_pieces and splits > 1:
@@ -1078,11 +1090,13 @@ def paged_attention(
             run(0, leading_single)
             run(leading_single, num_requests)
         else:
-            pieces = run(0, num_requests, leave_pieces=not combine and sink_logit is None and leading_single == num_requests)
+            pieces = run(0, num_requests, leave_pieces=not combine and sink_logit is None and chunk is None
+                         and leading_single == num_requests)
             if pieces is not None:
                 return pieces
         return out
 
+    assert chunk is None  # (a chunked mask on plain pages has gone to the general entry point above)
     splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)
     part_acc, part_ml = partials(splits)
     library.check(
@@ -1104,7 +1118,7 @@ def _paged_attention_general(
     q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor | None, block_table: torch.Tensor,
     token_request: torch.Tensor, positions: torch.Tensor, *, q_heads: int, kv_heads: int, head_dim: int,
     v_head_dim: int, scale: float, window: int | None, max_seq_len: int, v_transposed: bool,
-    slopes: torch.Tensor | None, sink_logit: float | None,
+    slopes: torch.Tensor | None, sink_logit: float | None, chunk: int | None = None,
 ) -> torch.Tensor:
     """The plain attention kernel with everything it can be told: see `paged_attention`."""
     _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, slopes)
@@ -1144,7 +1158,8 @@ def _paged_attention_general(
         raise KernelShapeError(f"slopes must be float32 [{q_heads}], got {slopes.dtype} x {slopes.numel()}")
     out = torch.empty((tokens, q_heads * v_head_dim), dtype=q.dtype, device=q.device)
     group = q_heads // kv_heads
-    splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)
+    # (no row sees more keys than a chunk holds)
+    splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), min(max_seq_len, chunk) if chunk else max_seq_len)
     part_acc = part_ml = None
     if splits > 1:
         part_acc = torch.empty((tokens * q_heads * splits, v_head_dim), dtype=torch.float32, device=q.device)
@@ -1154,7 +1169,7 @@ def _paged_attention_general(
             _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(values), _ptr(block_table), block_table.shape[1],
             _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), tokens,
             q_heads, kv_heads, head_dim, v_head_dim, v_row_stride, page_size, num_pages, float(scale), int(window or 0),
-            splits, _ptr(slopes), int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
+            splits, _ptr(slopes), int(sink_logit is not None), float(sink_logit or 0.0), int(chunk or 0), _stream(),
         )
     )
     return out
@@ -1585,16 +1600,20 @@ def linear_clamped_glu(x: torch.Tensor, gate_up_weight: torch.Tensor, bias: torc
 
 def short_conv(
     x: torch.Tensor, channels: int, taps_weight: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
-    slots: torch.Tensor, token_request: torch.Tensor,
+    slots: torch.Tensor, token_request: torch.Tensor, bias: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """A causal convolution over time per channel, then silu, on the first `channels` columns of
-    `x` [T, >= channels]: `y[t, c] = silu(sum_j w[c, j] * x[t - (taps-1) + j, c])` within each
+    `x` [T, >= channels]: `y[t, c] = silu(bias[c] + sum_j w[c, j] * x[t - (taps-1) + j, c])` within each
     request.  `tail` [slots + 1, taps - 1, channels] (compute dtype, rows may be strided) holds
     each request's last taps-1 inputs and is advanced in place; `taps_weight` is float32
     [channels, taps], last column the current token's."""
-    _need_cuda(x, taps_weight, tail, cu_seqlens, slots, token_request)
-    for name, t in (("taps_weight", taps_weight), ("cu_seqlens", cu_seqlens), ("slots", slots), ("token_request", token_request)):
+    _need_cuda(x, taps_weight, tail, cu_seqlens, slots, token_request, bias)
+    for name, t in (("taps_weight", taps_weight), ("cu_seqlens", cu_seqlens), ("slots", slots), ("token_request", token_request),
+                    ("bias", bias)):
         _need_contiguous(name, t)
+    _need_f32("bias", bias)
+    if bias is not None and bias.numel() != channels:
+        raise KernelShapeError(f"short_conv: the bias has {bias.numel()} entries for {channels} channels")
     for name, t in (("cu_seqlens", cu_seqlens), ("slots", slots), ("token_request", token_request)):
         _need_int32(name, t)
     _need_f32("taps_weight", taps_weight)
@@ -1614,7 +1633,7 @@ def short_conv(
     library.check(
         library.load().mi_short_conv(
             _dtype_code(x), _ptr(x), x.stride(0), _ptr(taps_weight), _ptr(tail), tail.stride(0), _ptr(cu_seqlens), _ptr(slots),
-            _ptr(token_request), _ptr(y), y.stride(0), tokens, requests, channels, taps, tail.shape[0] - 1, _stream(),
+            _ptr(token_request), _ptr(y), y.stride(0), tokens, requests, channels, taps, tail.shape[0] - 1, _ptr(bias), _stream(),
         )
     )
     return y
@@ -1834,3 +1853,274 @@ def sample_slots(logits: torch.Tensor, slots: torch.Tensor, slot_table: torch.Te
         )
     )
     return out
+
+
+# ----------------------------------------------------------------------------
+# a stream kept in several copies; recurrences with a decaying matrix state; heads normed one by one
+# ----------------------------------------------------------------------------
+
+MAX_STREAM_COPIES = 8
+
+
+def embed_norm_streams(table: torch.Tensor, ids: torch.Tensor, weight: torch.Tensor, copies: int, eps: float) -> torch.Tensor:
+    """`x = table[ids]`, divided by its root mean square (eps inside the root), times `weight`
+    (float32 [H], the factor itself), written `copies` times: float32 [T, copies, H]."""
+    _need_cuda(table, ids, weight)
+    for name, t in (("table", table), ("ids", ids), ("weight", weight)):
+        _need_contiguous(name, t)
+    _need_int32("ids", ids)
+    _need_f32("weight", weight)
+    vocab, hidden = table.shape
+    if weight.numel() != hidden or not 1 <= copies <= MAX_STREAM_COPIES:
+        raise KernelShapeError(f"embed_norm_streams: weight of {weight.numel()} for {hidden} columns, {copies} copies (1..{MAX_STREAM_COPIES})")
+    out = torch.empty((ids.numel(), copies, hidden), dtype=torch.float32, device=table.device)
+    library.check(
+        library.load().mi_embed_norm_streams(
+            _dtype_code(table), _ptr(table), _ptr(ids), _ptr(weight), _ptr(out), ids.numel(), hidden, vocab, copies, float(eps),
+            _stream(),
+        )
+    )
+    return out
+
+
+@dataclasses.dataclass
+class StreamsWrite:
+    """A sublayer's write into a stream kept in S copies that has not been made yet:
+
+        y = scale_a * a + scale_b * b;      x_t <- sum_s mix[s, t] * x_s + out[t] * y      (all copies at once)
+
+    `a`, `b`: sublayer outputs [T, H] in the compute dtype (`b` may be None); `mix` float32 [S, S]
+    indexed [from, to], `out` float32 [S].  A norm that knows it makes the write together with
+    the next read and its own statistics in one launch (`streams_update_norm`); `apply(streams)`
+    makes the write alone."""
+
+    a: torch.Tensor
+    mix: torch.Tensor
+    out: torch.Tensor
+    b: torch.Tensor | None = None
+    scale_a: float = 1.0
+    scale_b: float = 1.0
+
+    def apply(self, streams: torch.Tensor) -> None:
+        streams_update_norm(self, streams, None, None, 0.0, self.a.dtype)
+
+
+def streams_update_norm(
+    write: StreamsWrite | None, streams: torch.Tensor, read: torch.Tensor | None, weight: torch.Tensor | None, eps: float,
+    dtype: torch.dtype, rows: torch.Tensor | None = None,
+) -> torch.Tensor | None:
+    """Make `write` on the float32 copies [T, S, H] in place (kept unless `rows`), then read them
+    as `u = sum_t read[t] * x_t` (`read` float32 [S]; None: the plain sum) and return
+    `u / rms(u) * weight` (`weight` float32 [H], the factor itself) in `dtype`: [T, H] or
+    [len(rows), H].  `weight=None`: the write alone."""
+    tensors = (streams, read, weight, rows) + ((write.a, write.b, write.mix, write.out) if write is not None else ())
+    _need_cuda(*tensors)
+    for name, t in (("streams", streams), ("read", read), ("weight", weight), ("rows", rows)):
+        _need_contiguous(name, t)
+    _need_int32("rows", rows)
+    for name, t in (("streams", streams), ("read", read), ("weight", weight)):
+        _need_f32(name, t)
+    if streams.dim() != 3 or not 1 <= streams.shape[1] <= MAX_STREAM_COPIES:
+        raise KernelShapeError(f"streams are float32 [T, copies <= {MAX_STREAM_COPIES}, H], got {tuple(streams.shape)}")
+    tokens, copies, hidden = streams.shape
+    if read is not None and read.numel() != copies:
+        raise KernelShapeError(f"the read vector has {read.numel()} entries for {copies} copies")
+    if weight is not None and weight.numel() != hidden:
+        raise KernelShapeError(f"the norm weight has {weight.numel()} entries for {hidden} columns")
+    if weight is None and rows is not None:
+        raise KernelShapeError("a row list only goes with a norm")
+    a = b = mix = out_vec = None
+    scale_a = scale_b = 1.0
+    if write is not None:
+        a, b, mix, out_vec, scale_a, scale_b = write.a, write.b, write.mix, write.out, write.scale_a, write.scale_b
+        _need_f32("mix", mix)
+        _need_f32("out", out_vec)
+        _need_contiguous("mix", mix)
+        _need_contiguous("out", out_vec)
+        if tuple(mix.shape) != (copies, copies) or out_vec.numel() != copies:
+            raise KernelShapeError(f"a write into {copies} copies needs mix [{copies}, {copies}] and out [{copies}]")
+        for name, t in (("a", a), ("b", b)):
+            if t is not None and (t.dim() != 2 or tuple(t.shape) != (tokens, hidden) or t.stride(1) != 1 or t.dtype != dtype):
+                raise KernelShapeError(f"streams write: {name} {tuple(t.shape)} {t.dtype} does not fit {(tokens, hidden)} in {dtype}")
+    n_out = tokens if rows is None else rows.numel()
+    result = torch.empty((n_out, hidden), dtype=dtype, device=streams.device) if weight is not None else None
+    library.check(
+        library.load().mi_streams_update_norm(
+            F32 if dtype == torch.float32 else BF16, _ptr(a), 0 if a is None else a.stride(0), _ptr(b),
+            0 if b is None else b.stride(0), float(scale_a), float(scale_b), _ptr(mix), _ptr(out_vec), _ptr(read), _ptr(weight),
+            _ptr(streams), _ptr(result), _ptr(rows), n_out, hidden, copies, float(eps), _stream(),
+        )
+    )
+    return result
+
+
+def decay_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int]:
+    """How `decay_scan` lays a request's state out: per head S transposed, [vdim][padded dim]."""
+    if dim > 256:
+        raise KernelShapeError(f"decay_scan takes key widths up to 256, got {dim}")
+    pad = 16 if dim <= 16 else (32 if dim <= 32 else (64 if dim <= 64 else (128 if dim <= 128 else 256)))
+    return (heads, vdim, pad)
+
+
+def decay_scan(
+    q: torch.Tensor, q_col: int, k: torch.Tensor, k_col: int, v: torch.Tensor, v_col: int, gate: torch.Tensor, gate_col: int,
+    gate_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, *, heads: int, groups: int,
+    dim: int, vdim: int, per_head: bool, rate: torch.Tensor | None = None, skip: torch.Tensor | None = None,
+    inv_tau: float = 1.0, q_scale: float = 1.0,
+) -> torch.Tensor:
+    """The recurrence `S <- diag(a) S + k v^T; o = S^T q` over the rows of a step, per request and
+    head, float32 state [slots + 1, *decay_state_shape(...)] advanced in place; returns the
+    read-outs float32 [T, heads*vdim].
+
+    `q`, `k`: rows that hold `groups` heads of `dim` from `q_col` / `k_col` on (head h reads
+    group h // (heads // groups)); `v`: rows that hold `heads` heads of `vdim` from `v_col` on.
+    `per_head=False`: `gate` rows hold heads*dim logits z from `gate_col` on and
+    `a = logistic(z + gate_bias) ** inv_tau`, q enters times `q_scale`.  `per_head=True`: `gate`
+    rows hold `heads` raw step sizes, `dt = softplus(raw + gate_bias)`, `a = exp(-exp(rate) * dt)`,
+    v enters times dt and the read-out gets `skip[h] * v` added."""
+    _need_cuda(q, k, v, gate, gate_bias, state, cu_seqlens, slots, rate, skip)
+    for name, t in (("gate_bias", gate_bias), ("cu_seqlens", cu_seqlens), ("slots", slots), ("rate", rate), ("skip", skip)):
+        _need_contiguous(name, t)
+    for name, t in (("gate_bias", gate_bias), ("rate", rate), ("skip", skip), ("state", state)):
+        _need_f32(name, t)
+    _need_int32("cu_seqlens", cu_seqlens)
+    _need_int32("slots", slots)
+    tokens = q.shape[0]
+    for name, t in (("q", q), ("k", k), ("v", v), ("gate", gate)):
+        if t.dim() != 2 or t.stride(1) != 1 or t.shape[0] != tokens or t.dtype != q.dtype:
+            raise KernelShapeError(f"decay_scan: {name} must be rows of the same step and dtype with unit inner stride")
+    if q.shape[1] < q_col + groups * dim or k.shape[1] < k_col + groups * dim or v.shape[1] < v_col + heads * vdim:
+        raise KernelShapeError("decay_scan: the q, k or v columns lie outside their rows")
+    gate_width = heads if per_head else heads * dim
+    if gate.shape[1] < gate_col + gate_width or gate_bias.numel() != gate_width:
+        raise KernelShapeError(f"decay_scan: the gates need {gate_width} columns and as many biases")
+    if per_head and (rate is None or rate.numel() != heads or (skip is not None and skip.numel() != heads)):
+        raise KernelShapeError("decay_scan: one rate (and one skip weight) per head")
+    shape = decay_state_shape(heads, dim, vdim)
+    if state.dim() != 4 or tuple(state.shape[1:]) != shape or state.shape[0] < 2 or not state[0].is_contiguous():
+        raise KernelShapeError(f"decay_scan: the state is float32 [slots + 1, {shape}] with packed slots, got {tuple(state.shape)}")
+    requests = slots.numel()
+    if cu_seqlens.numel() != requests + 1:
+        raise KernelShapeError("decay_scan: one more boundary than requests")
+    out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=q.device)
+    library.check(
+        library.load().mi_decay_scan(
+            _dtype_code(q), int(per_head), _ptr(q), q.stride(0), int(q_col), _ptr(k), k.stride(0), int(k_col), _ptr(v),
+            v.stride(0), int(v_col), _ptr(gate), gate.stride(0), int(gate_col), _ptr(gate_bias), _ptr(rate), _ptr(skip),
+            float(inv_tau), float(q_scale), _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(slots), state.shape[0] - 1,
+            _ptr(out), tokens, requests, heads, groups, dim, vdim, _stream(),
+        )
+    )
+    return out
+
+
+def readout_gate_norm(
+    readout: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, *, group_width: int, gate_first: bool, eps: float,
+) -> torch.Tensor:
+    """What follows a recurrence's read-outs (float32 [T, W]): an RMS norm over groups of
+    `group_width` columns times `weight` (float32; column c takes `weight[c % len(weight)]`) and
+    the gate `silu(gate)` ([T, W] in the compute dtype, rows may be strided).  `gate_first`:
+    `norm(o * silu(g)) * w`, else `norm(o) * w * silu(g)`.  Returns [T, W] in the gate's dtype."""
+    _need_cuda(readout, gate, weight)
+    _need_contiguous("readout", readout)
+    _need_contiguous("weight", weight)
+    _need_f32("readout", readout)
+    _need_f32("weight", weight)
+    tokens, width = readout.shape
+    if gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != tokens or gate.shape[1] < width:
+        raise KernelShapeError(f"readout_gate_norm: the gate must be [T, >= {width}] with unit inner stride")
+    if width % group_width != 0 or width % weight.numel() != 0:
+        raise KernelShapeError(f"readout_gate_norm: {width} columns in groups of {group_width} with a weight of {weight.numel()}")
+    out = torch.empty((tokens, width), dtype=gate.dtype, device=gate.device)
+    library.check(
+        library.load().mi_readout_gate_norm(
+            _dtype_code(gate), _ptr(readout), _ptr(gate), gate.stride(0), _ptr(weight), weight.numel(), _ptr(out), out.stride(0),
+            tokens, width, int(group_width), int(gate_first), float(eps), _stream(),
+        )
+    )
+    return out
+
+
+def head_norm_rope_kv_write(
+    qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, slot_mapping: torch.Tensor | None, k_pages: torch.Tensor | None,
+    v_pages: torch.Tensor | None, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None, eps: float, *, q_heads: int,
+    kv_heads: int, head_dim: int, rotary_dim: int, interleaved: bool = False, v_transposed: bool = False,
+    v_head_dim: int | None = None,
+) -> None:
+    """`rope_kv_write` with every query and key head first divided by its own root mean square
+    over the head and multiplied by `q_weight` / `k_weight` (float32 [head_dim], shared by the
+    heads; None: that side is not normed)."""
+    _need_cuda(qkv, cos, sin, slot_mapping, k_pages, v_pages, q_weight, k_weight)
+    for name, t in (("cos", cos), ("sin", sin), ("slot_mapping", slot_mapping), ("k_pages", k_pages), ("v_pages", v_pages),
+                    ("q_weight", q_weight), ("k_weight", k_weight)):
+        _need_contiguous(name, t)
+    _need_int32("slot_mapping", slot_mapping)
+    _need_f32("q_weight", q_weight)
+    _need_f32("k_weight", k_weight)
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise KernelShapeError(f"qkv must be [T, width] with unit inner stride, got {qkv.stride()}")
+    tokens = qkv.shape[0]
+    v_dim = head_dim if v_head_dim is None else int(v_head_dim)
+    if qkv.shape[1] < (q_heads + kv_heads) * head_dim + kv_heads * v_dim:
+        raise KernelShapeError("qkv rows hold fewer values than the q, k and v heads need")
+    if cos.shape != (tokens, rotary_dim // 2) or sin.shape != cos.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+        raise KernelShapeError(f"cos/sin must be float32 [{tokens}, {rotary_dim // 2}], got {tuple(cos.shape)} {cos.dtype}")
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if t is not None and t.numel() != head_dim:
+            raise KernelShapeError(f"{name} has {t.numel()} entries for heads of {head_dim}")
+    page_size = num_pages = 0
+    if kv_heads > 0 and slot_mapping is not None:
+        if k_pages is None or v_pages is None:
+            raise KernelShapeError("writing keys and values needs k_pages and v_pages")
+        if k_pages.dtype != qkv.dtype or v_pages.dtype != qkv.dtype:
+            raise KernelShapeError(f"pages are {k_pages.dtype}, activations {qkv.dtype}")
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelShapeError(f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}")
+        _check_v_pages(k_pages, v_pages, v_transposed, v_dim)
+        if slot_mapping.numel() != tokens:
+            raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    library.check(
+        library.load().mi_head_norm_rope_kv_write(
+            _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(cos), _ptr(sin), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages),
+            _ptr(q_weight), _ptr(k_weight), float(eps), tokens, q_heads, kv_heads, head_dim, rotary_dim, int(interleaved),
+            page_size, num_pages, int(v_transposed), v_dim, _stream(),
+        )
+    )
+
+
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "logistic": 2}
+
+
+def gated_mul(a: torch.Tensor, b: torch.Tensor, activation: str) -> torch.Tensor:
+    """`act(a) * b` elementwise for [T, W] column ranges of rows (rows may be strided):
+    `silu`, `gelu_tanh` (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or `logistic`."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelShapeError(f"gated_mul: activation {activation!r}; built: {sorted(GATE_ACTIVATIONS)}")
+    _need_cuda(a, b)
+    if a.dim() != 2 or a.shape != b.shape or a.stride(1) != 1 or b.stride(1) != 1 or a.dtype != b.dtype:
+        raise KernelShapeError(f"gated_mul: two [T, W] ranges of one dtype with unit inner stride, got {tuple(a.shape)} {tuple(b.shape)}")
+    tokens, width = a.shape
+    out = torch.empty((tokens, width), dtype=a.dtype, device=a.device)
+    library.check(
+        library.load().mi_gated_mul(
+            _dtype_code(a), GATE_ACTIVATIONS[activation], _ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(out), out.stride(0),
+            tokens, width, _stream(),
+        )
+    )
+    return out
+
+
+@dataclasses.dataclass
+class WeightedSum:
+    """`scale_a * a + scale_b * b` of two sublayer outputs [T, H] in the compute dtype, not made
+    yet: a stream write that knows it (`StreamsWrite`) makes it on its way; anything else calls
+    `finish()`."""
+
+    a: torch.Tensor
+    b: torch.Tensor
+    scale_a: float = 1.0
+    scale_b: float = 1.0
+
+    def finish(self) -> torch.Tensor:
+        return (self.scale_a * self.a.float() + self.scale_b * self.b.float()).to(self.a.dtype)

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 29
+ABI_VERSION = 30
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -57,7 +57,7 @@ _SIGNATURES: dict[str, list] = {
     ],
     "mi_attn_mfma": [
         _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
-        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P,
+        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
     ],
     "mi_gemm_skinny_addnorm_pieces": [c_int],
     "mi_gemm_skinny_addnorm_bf16": [
@@ -80,11 +80,11 @@ _SIGNATURES: dict[str, list] = {
     "mi_gated_table_rows": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
     "mi_attn_general": [
         c_int, _P, c_int64, _P, _P, _P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, c_int,
-        c_int64, c_int, c_int, c_float, c_int, c_int, _P, c_int, c_float, _P,
+        c_int64, c_int, c_int, c_float, c_int, c_int, _P, c_int, c_float, c_int, _P,
     ],
     "mi_stream_update_norm": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_float, _P],
     "mi_clamped_glu": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_float, _P],
-    "mi_short_conv": [c_int, _P, c_int64, _P, _P, c_int64, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P],
+    "mi_short_conv": [c_int, _P, c_int64, _P, _P, c_int64, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P, _P],
     "mi_gated_delta": [
         c_int, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int64,
         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
@@ -98,6 +98,21 @@ _SIGNATURES: dict[str, list] = {
         c_int, _P, c_int64, c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
         c_int, _P,
     ],
+    "mi_embed_norm_streams": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
+    "mi_streams_update_norm": [
+        c_int, _P, c_int64, _P, c_int64, c_float, c_float, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P,
+    ],
+    "mi_decay_scan_dim_pad": [c_int],
+    "mi_decay_scan": [
+        c_int, c_int, _P, c_int64, c_int, _P, c_int64, c_int, _P, c_int64, c_int, _P, c_int64, c_int, _P, _P, _P, c_float,
+        c_float, _P, c_int64, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P,
+    ],
+    "mi_readout_gate_norm": [c_int, _P, _P, c_int64, _P, c_int, _P, c_int64, c_int, c_int, c_int, c_int, c_float, _P],
+    "mi_head_norm_rope_kv_write": [
+        c_int, _P, c_int64, _P, _P, _P, _P, _P, _P, _P, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+        c_int, c_int, _P,
+    ],
+    "mi_gated_mul": [c_int, c_int, _P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, _P],
 }
 
 

@@ -5,7 +5,10 @@ Order of operations as in the reference's `GroupedQueryAttention.forward`
 q and k fused with the write of k and v into cache pages
 (rope_write_kernel.py:75-152), causal attention over the pages with scale
 1/sqrt(head_dim) (cache/packed_attention.py:126-127, :296-338), output
-projection.  A window, if given, limits each query to the last `window` keys.
+projection.  A window, if given, limits each query to the last `window` keys; a chunk to
+the keys of its own stretch of `chunk` positions.  Queries and keys may be normed head by
+head before the rotation, and the attended rows may be gated by a projection of the
+layer's input before the output projection.
 """
 
 from __future__ import annotations
@@ -50,15 +53,38 @@ class GQAttention(Mixer):
         suffix: str = ".weight",
         v_head_dim: int | None = None,
         sink_logit: float | None = None,
+        chunk: int | None = None,
+        head_norm: dict | None = None,
+        gate: dict | None = None,
     ) -> None:
         """`v_head_dim`: value heads of another width than the query and key heads (`head_dim`).
         `sink_logit`: the softmax's denominator gets one more term exp(sink_logit), a sink that
-        takes weight off the keys and carries no value (0.0: the denominator grows by exp(0) = 1)."""
+        takes weight off the keys and carries no value (0.0: the denominator grows by exp(0) = 1).
+        `chunk`: position i sees j <= i only if i // chunk == j // chunk (chunks are counted from
+        position 0 of the sequence, wherever a prompt was cut).
+        `head_norm` = {"eps": e, "names": (q_name, k_name)}: every query head and every key head is
+        divided by its own root mean square over the head and multiplied by a weight of `head_dim`
+        entries that the heads share, before the rotation.
+        `gate` = {"name": n, "activation": "logistic"}: one more projection of the layer's input, as wide as
+        the concatenated value heads; the attended rows are multiplied by its activation, element
+        by element, before the output projection."""
         super().__init__(dtype, device)
         if num_heads % num_kv_heads != 0:
             raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
         if window is not None and window <= 0:
             raise ValueError(f"window must be positive, got {window}")
+        if chunk is not None and chunk <= 0:
+            raise ValueError(f"chunk must be positive, got {chunk}")
+        self.chunk = None if chunk is None else int(chunk)
+        self.head_norm_eps = None if head_norm is None else float(head_norm["eps"])
+        self.head_norm_names = None if head_norm is None else tuple(head_norm.get("names", ("q_norm", "k_norm")))
+        self.gate_name = None if gate is None else str(gate["name"])
+        self.gate_activation = None if gate is None else str(gate.get("activation", "logistic"))
+        # the few-row kernels that fold projection, rotation and cache write (and the output
+        # projection's hand-over) know neither head norms nor gates
+        self._plain_heads = head_norm is None and gate is None
+        self.q_norm_weight: torch.Tensor | None = None
+        self.k_norm_weight: torch.Tensor | None = None
         if head_dim <= 0 or head_dim % ops.ATTENTION_HEAD_DIM_STEP != 0 or head_dim > ops.ATTENTION_MAX_HEAD_DIM:
             raise ValueError(
                 f"head_dim={head_dim}: the attention kernels take even head sizes "
@@ -90,14 +116,25 @@ class GQAttention(Mixer):
     def _input_projection(self, hidden_size: int, q_width: int, kv_width: int, names, suffix: str) -> Linear:
         """The stacked product that feeds the attention: q | k | v here."""
         v_width = self.num_kv_heads * self.v_head_dim
-        return Linear(hidden_size, [q_width, kv_width, v_width], list(names[:3]), self.dtype, self.device, suffix=suffix)
+        widths, parts = [q_width, kv_width, v_width], list(names[:3])
+        if self.gate_name is not None:  # q | k | v | gate
+            widths.append(self.num_heads * self.v_head_dim)
+            parts.append(self.gate_name)
+        return Linear(hidden_size, widths, parts, self.dtype, self.device, suffix=suffix)
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
-        return {**self.qkv.param_specs(prefix), **self.out.param_specs(prefix)}
+        specs = {**self.qkv.param_specs(prefix), **self.out.param_specs(prefix)}
+        if self.head_norm_names is not None:
+            for name in self.head_norm_names:
+                specs[prefix + name] = ParamSpec((self.head_dim,), init="norm_weight", dtype="float32")
+        return specs
 
     def load_params(self, prefix: str, get: TensorGetter) -> None:
         self.qkv.load_params(prefix, get)
         self.out.load_params(prefix, get)
+        if self.head_norm_names is not None:
+            self.q_norm_weight = get(prefix + self.head_norm_names[0]).float().contiguous()
+            self.k_norm_weight = get(prefix + self.head_norm_names[1]).float().contiguous()
 
     def wants_scaled_rows(self, rows: int) -> bool:
         """Only where projection, rotation and cache write will run as the one kernel that
@@ -106,6 +143,7 @@ class GQAttention(Mixer):
         return (
             self.dtype == torch.bfloat16
             and self._same_widths
+            and self._plain_heads
             and layout == (self.head_dim, False)
             and self.head_dim % 32 == 0
             and ops.scaled_rows_product_takes(rows, self.qkv.weight, self.hidden_size)
@@ -133,10 +171,11 @@ class GQAttention(Mixer):
         if isinstance(x, ops.ScaledRows) and not (
             rotary is not None
             and self._same_widths
+            and self._plain_heads
             and ops.qkv_rope_write_takes(x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved)
         ):
             x = x.finish()  # rows but for their norm factors, and no kernel here that applies them
-        if rotary is not None and self._same_widths and ops.qkv_rope_write_takes(
+        if rotary is not None and self._same_widths and self._plain_heads and ops.qkv_rope_write_takes(
             x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved
         ):
             # few rows (decode): projection, rotation and cache write are one kernel
@@ -160,13 +199,30 @@ class GQAttention(Mixer):
         else:
             cos = sin = torch.empty((ctx.num_tokens, 0), dtype=torch.float32, device=x.device)
             rotary_dim, interleaved = 0, False
-        ops.rope_kv_write(
-            qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
-            q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
-            rotary_dim=rotary_dim, interleaved=interleaved, v_transposed=cache.v_transposed,
-            v_head_dim=self.v_head_dim,
-        )
-        return self._project(self._attend(qkv, ctx, cache))
+        if self.head_norm_eps is not None:
+            assert self.q_norm_weight is not None, "attention used before its weights were loaded"
+            ops.head_norm_rope_kv_write(
+                qkv, cos, sin, slots, cache.k_pages, cache.v_pages, self.q_norm_weight,
+                self.k_norm_weight if writes_cache else None, self.head_norm_eps,
+                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+                rotary_dim=rotary_dim, interleaved=interleaved, v_transposed=cache.v_transposed,
+                v_head_dim=self.v_head_dim,
+            )
+        else:
+            ops.rope_kv_write(
+                qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
+                q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
+                rotary_dim=rotary_dim, interleaved=interleaved, v_transposed=cache.v_transposed,
+                v_head_dim=self.v_head_dim,
+            )
+        attended = self._attend(qkv, ctx, cache)
+        if self.gate_name is not None:
+            if not writes_cache:
+                raise NotImplementedError("a gated attention layer that reads another call's keys projects its own gate; not built")
+            width = self.num_heads * self.v_head_dim
+            first = (self.num_heads + self.num_kv_heads) * self.head_dim + self.num_kv_heads * self.v_head_dim
+            attended = ops.gated_mul(qkv[:, first:first + width], attended, self.gate_activation)
+        return self._project(attended)
 
     def _project(self, attended):
         """The output projection of what `_attend` returned; for few rows, where the block
@@ -187,6 +243,7 @@ class GQAttention(Mixer):
         projection to combine on its way (one launch less a layer)."""
         few = (
             queries.dtype == torch.bfloat16 and self._same_widths and self.sink_logit is None
+            and self._plain_heads and self.chunk is None
             and ops.attention_pieces_pay(ctx.num_tokens, self.num_heads, self.head_dim)
         )
         return ops.paged_attention(
@@ -194,7 +251,7 @@ class GQAttention(Mixer):
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few, slopes=self.slopes,
-            v_head_dim=self.v_head_dim, sink_logit=self.sink_logit,
+            v_head_dim=self.v_head_dim, sink_logit=self.sink_logit, chunk=self.chunk,
         )
 
 
@@ -283,7 +340,7 @@ def build_gqa_attention(desc: dict, dtype: torch.dtype, device, shared: dict | N
             position = POSITION_ENCODINGS.lookup(pos_desc["kind"])(pos_desc, dtype, device, shared)
             if shared is not None:
                 shared[key] = position
-    extra = {k: desc[k] for k in ("suffix", "v_head_dim", "sink_logit") if k in desc}
+    extra = {k: desc[k] for k in ("suffix", "v_head_dim", "sink_logit", "chunk", "head_norm", "gate") if k in desc}
     if "names" in desc:
         extra["names"] = tuple(desc["names"])
     return GQAttention(

@@ -286,3 +286,99 @@ def build_output_norm_block(desc: dict, dtype: torch.dtype, device, shared: dict
         build(FEED_FORWARDS, side), build(NORMS, desc.get("side_norm")) if side is not None else None,
         int(desc["hidden_size"]), bool(desc.get("layer_scale", False)), dict(desc["names"]), dtype, device,
     )
+
+
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers around a residual stream that is kept in S copies x_1 .. x_S
+    (float32 [T, S, H]).  Sublayer q (the mixer, then the feed-forward if the layer has one) has
+    a read vector, a write vector and a matrix of its own:
+
+        u = sum_s in_q[s] x_s;    y = sublayer(norm_q(u));    x_t <- sum_s mix_q[s, t] x_s + out_q[t] y
+
+    (every copy rewritten at once from the old ones).  Without learned vectors (`learned=False`)
+    there is one copy, read as it is and written by a plain add: the usual pre-norm layer.
+
+    The norms are `streams_rms_norm`s: each makes the write the sublayer before it left, its own
+    read and its statistics in one launch, so the block's last write is handed on as
+    `ops.StreamsWrite` to whatever norm comes next."""
+
+    takes_pending_products = False
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, feed_forward: FeedForward | None, copies: int,
+                 learned: bool, names: dict[str, str], dtype: torch.dtype, device) -> None:
+        super().__init__(dtype, device)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward = mixer_norm, mixer, ffn_norm, feed_forward
+        self.copies, self.learned, self.names = int(copies), bool(learned), names
+        if not learned and copies != 1:
+            raise ValueError("a stream in several copies needs its read and write vectors")
+        self.vectors: dict[str, torch.Tensor] = {}
+
+    def _children(self):
+        parts = [(self.names["mixer_norm"], self.mixer_norm), (self.names["mixer"], self.mixer)]
+        if self.feed_forward is not None:
+            parts += [(self.names["ffn_norm"], self.ffn_norm), (self.names["feed_forward"], self.feed_forward)]
+        return parts
+
+    def _connections(self) -> list[str]:
+        return [self.names["mixer_connection"]] + ([self.names["ffn_connection"]] if self.feed_forward is not None else [])
+
+    @property
+    def graph_safe(self) -> bool:  # type: ignore[override]
+        return all(part.graph_safe for _, part in self._children())
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        specs: dict[str, ParamSpec] = {}
+        for sub, part in self._children():
+            specs.update(part.param_specs(prefix + sub))
+        if self.learned:
+            S = self.copies
+            for sub in self._connections():
+                specs[prefix + sub + "in"] = ParamSpec((S,), init="norm_weight", dtype="float32")
+                specs[prefix + sub + "out"] = ParamSpec((S,), init="norm_weight", dtype="float32")
+                specs[prefix + sub + "mix"] = ParamSpec((S, S), init="norm_weight", dtype="float32")
+        return specs
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        for sub, part in self._children():
+            part.load_params(prefix + sub, get)
+        for sub in self._connections():
+            for what in ("in", "out", "mix"):
+                if self.learned:
+                    self.vectors[sub + what] = get(prefix + sub + what).float().contiguous()
+                else:
+                    shape = (1, 1) if what == "mix" else (1,)
+                    self.vectors[sub + what] = torch.ones(shape, dtype=torch.float32, device=self.device)
+        self.mixer_norm.read = self.vectors[self.names["mixer_connection"] + "in"] if self.learned else None
+        if self.ffn_norm is not None:
+            self.ffn_norm.read = self.vectors[self.names["ffn_connection"] + "in"] if self.learned else None
+
+    def _write(self, y, connection: str):
+        from mini_infer_amd import ops
+
+        mix, out = self.vectors[connection + "mix"], self.vectors[connection + "out"]
+        if isinstance(y, ops.WeightedSum):
+            return ops.StreamsWrite(y.a, mix, out, b=y.b, scale_a=y.scale_a, scale_b=y.scale_b)
+        return ops.StreamsWrite(y.finish() if hasattr(y, "finish") else y, mix, out)
+
+    def forward(self, delta, residual: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        h = self.mixer_norm.forward(delta, residual)
+        pending = self._write(self.mixer.forward(h, ctx, cache, writes_cache), self.names["mixer_connection"])
+        if self.feed_forward is None:
+            return pending
+        h = self.ffn_norm.forward(pending, residual)
+        return self._write(self.feed_forward.forward(h, ctx), self.names["ffn_connection"])
+
+
+@register_block("hyper_connections")
+def build_hyper_connection_block(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> HyperConnectionBlock:
+    """`desc`: `norm` (for both sublayers), `mixer`, optional `feed_forward`, `copies`, `learned`
+    (whether the layer has read and write vectors of its own) and `names`."""
+    shared = {} if shared is None else shared
+    ffn = desc.get("feed_forward")
+    return HyperConnectionBlock(
+        NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype, device, shared),
+        MIXERS.lookup(desc["mixer"]["kind"])(desc["mixer"], dtype, device, shared),
+        NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype, device, shared) if ffn is not None else None,
+        FEED_FORWARDS.lookup(ffn["kind"])(ffn, dtype, device, shared) if ffn is not None else None,
+        int(desc.get("copies", 1)), bool(desc.get("learned", True)), dict(desc["names"]), dtype, device,
+    )

@@ -169,3 +169,35 @@ def build_linear_head(desc: dict, dtype: torch.dtype, device, shared: dict | Non
     return OutputHead(
         int(desc["hidden_size"]), int(desc["vocab_size"]), str(desc["name"]), dtype, device, tied_to=tied_to
     )
+
+
+class NormedStreamsEmbedding(TokenEmbedding):
+    """`table[token]` divided by its root mean square and multiplied by `offset + w` (`w` of its
+    own: `norm_name`), written `copies` times: the start of a residual stream that is kept in
+    several copies, float32 [T, copies, H]."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, norm_name: str, eps: float, copies: int,
+                 dtype: torch.dtype, device, weight_offset: float = 0.0) -> None:
+        super().__init__(vocab_size, hidden_size, name, dtype, device)
+        self.norm_name, self.eps, self.copies, self.weight_offset = norm_name, float(eps), int(copies), float(weight_offset)
+        self.factor: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        init = "norm_weight" if self.weight_offset == 0.0 else "normal"
+        return {**super().param_specs(prefix), prefix + self.norm_name: ParamSpec((self.hidden_size,), init=init, dtype="float32")}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        super().load_params(prefix, get)
+        self.factor = (get(prefix + self.norm_name).float() + self.weight_offset).contiguous()
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        assert self.weight is not None and self.factor is not None, "embedding used before its tensors were loaded"
+        return ops.embed_norm_streams(self.weight, ctx.token_ids, self.factor, self.copies, self.eps)
+
+
+@register_embedding("normed_streams_embedding")
+def build_normed_streams_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> NormedStreamsEmbedding:
+    return NormedStreamsEmbedding(
+        int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), str(desc["norm_name"]), float(desc["eps"]),
+        int(desc.get("copies", 1)), dtype, device, weight_offset=float(desc.get("weight_offset", 0.0)),
+    )

@@ -1,4 +1,5 @@
-"""Dense gated feed-forward: `down(silu(gate(x)) * up(x))`, no biases.
+"""Dense gated feed-forward: `down(act(gate(x)) * up(x))`, no biases; act is silu unless a
+layer's description says otherwise (the tanh form of gelu is the other one built).
 
 Formula: models/blocks/swiglu.py:44-46 and activations.py:36-45 of the
 reference.  Gate and up are two tensors in the checkpoint; they are stacked at
@@ -22,14 +23,22 @@ class SwiGLU(FeedForward):
     takes_scaled_rows = True
     can_defer_output = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, dtype: torch.dtype, device) -> None:
+    ACTIVATIONS = ("silu", "gelu_tanh")
+
+    def __init__(self, hidden_size: int, intermediate_size: int, dtype: torch.dtype, device, *, activation: str = "silu",
+                 names: tuple[str, str, str] = ("gate_proj", "up_proj", "down_proj"), suffix: str = ".weight") -> None:
         super().__init__(dtype, device)
+        if activation not in self.ACTIVATIONS:
+            raise NotImplementedError(f"gated feed-forward activation {activation!r}; built: {self.ACTIVATIONS}")
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        self.activation = activation
         self.gate_up = Linear(
-            hidden_size, [intermediate_size, intermediate_size], ["gate_proj", "up_proj"], dtype, device
+            hidden_size, [intermediate_size, intermediate_size], [names[0], names[1]], dtype, device, suffix=suffix
         )
-        self.down = Linear(intermediate_size, hidden_size, "down_proj", dtype, device)
+        self.down = Linear(intermediate_size, hidden_size, names[2], dtype, device, suffix=suffix)
+        if activation != "silu":  # the kernels that fold a norm's factors or the down product in are silu's
+            self.takes_scaled_rows = False
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
         return {**self.gate_up.param_specs(prefix), **self.down.param_specs(prefix)}
@@ -40,12 +49,19 @@ class SwiGLU(FeedForward):
 
     def wants_scaled_rows(self, rows: int) -> bool:
         """Where the gated product runs as the weight-streaming kernel that applies the rows' factors."""
-        return self.dtype == torch.bfloat16 and ops.scaled_rows_product_takes(rows, self.gate_up.weight, self.hidden_size)
+        return (self.activation == "silu" and self.dtype == torch.bfloat16
+                and ops.scaled_rows_product_takes(rows, self.gate_up.weight, self.hidden_size))
 
     def forward(self, x: "torch.Tensor | ops.ScaledRows", ctx: StepContext) -> torch.Tensor:
         assert self.gate_up.weight is not None, "SwiGLU used before its weights were loaded"
         assert self.down.weight is not None
-        act = ops.linear_swiglu(x, self.gate_up.weight)
+        if self.activation == "silu":
+            act = ops.linear_swiglu(x, self.gate_up.weight)
+        else:
+            if isinstance(x, ops.ScaledRows):
+                x = x.finish()
+            both = self.gate_up.forward(x)
+            act = ops.gated_mul(both[:, : self.intermediate_size], both[:, self.intermediate_size :], self.activation)
         if (
             self.emit_pending_output
             and self.dtype == torch.bfloat16
@@ -59,10 +75,10 @@ class SwiGLU(FeedForward):
 
 @register_feed_forward("swiglu")
 def build_swiglu(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> SwiGLU:
-    activation = desc.get("activation", "silu")
-    if activation != "silu":
-        raise NotImplementedError(f"gated feed-forward activation {activation!r}; only 'silu' is built")
-    return SwiGLU(int(desc["hidden_size"]), int(desc["intermediate_size"]), dtype, device)
+    extra = {k: desc[k] for k in ("activation", "suffix") if k in desc}
+    if "names" in desc:
+        extra["names"] = tuple(desc["names"])
+    return SwiGLU(int(desc["hidden_size"]), int(desc["intermediate_size"]), dtype, device, **extra)
 
 
 class PolyNormFeedForward(FeedForward):

@@ -113,3 +113,53 @@ class ScalarGainRMSNorm(Norm):
 @register_norm("scalar_rms_norm")
 def build_scalar_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ScalarGainRMSNorm:
     return ScalarGainRMSNorm(int(desc["hidden_size"]), float(desc["eps"]), dtype, device, name=str(desc.get("name", "weight")))
+
+
+class StreamsRMSNorm(Norm):
+    """RMS norm in front of a sublayer of a model whose residual stream is kept in several copies
+    x_1 .. x_S (float32 [T, S, H]).  It reads `u = sum_s read[s] * x_s` (no `read`: the plain
+    sum, which is how such a model ends) and returns `u / sqrt(mean(u^2) + eps) * (offset + w)`:
+    `weight_offset=1.0` is a weight stored around zero.
+
+    What the sublayer before it left to be written comes as `ops.StreamsWrite` (the copies are
+    rewritten all at once from the old ones through a small matrix, plus the sublayer's output
+    times a vector); write, read and norm are one launch.  `read` is set by the block that owns
+    the vectors."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, eps: float, copies: int, dtype: torch.dtype, device, name: str = "weight",
+                 weight_offset: float = 0.0) -> None:
+        super().__init__(dtype, device)
+        if not 1 <= copies <= ops.MAX_STREAM_COPIES:
+            raise ValueError(f"a stream is kept in 1..{ops.MAX_STREAM_COPIES} copies, got {copies}")
+        self.hidden_size, self.eps, self.copies = hidden_size, float(eps), int(copies)
+        self.name, self.weight_offset = name, float(weight_offset)
+        self.factor: torch.Tensor | None = None  # float32 [H]: offset + weight
+        self.read: torch.Tensor | None = None  # float32 [S], or None for the plain sum
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        init = "norm_weight" if self.weight_offset == 0.0 else "normal"
+        return {prefix + self.name: ParamSpec((self.hidden_size,), init=init, dtype="float32")}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.factor = (get(prefix + self.name).float() + self.weight_offset).contiguous()
+
+    def forward(self, delta, residual: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
+        assert self.factor is not None, "norm used before its weight was loaded"
+        if residual.dim() != 3 or residual.shape[1] != self.copies:
+            raise ValueError(f"this norm reads a stream of {self.copies} copies [T, {self.copies}, H], got {tuple(residual.shape)}")
+        if delta is not None and not isinstance(delta, ops.StreamsWrite):
+            if self.copies != 1:
+                raise TypeError("a stream kept in several copies is written through `ops.StreamsWrite` only")
+            # one copy: a plain residual add
+            delta = delta.finish() if hasattr(delta, "finish") else delta
+            one = torch.ones(1, dtype=torch.float32, device=residual.device)
+            delta = ops.StreamsWrite(delta, one.reshape(1, 1), one)
+        return ops.streams_update_norm(delta, residual, self.read, self.factor, self.eps, self.dtype, rows)
+
+
+@register_norm("streams_rms_norm")
+def build_streams_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> StreamsRMSNorm:
+    return StreamsRMSNorm(int(desc["hidden_size"]), float(desc["eps"]), int(desc.get("copies", 1)), dtype, device,
+                          name=str(desc.get("name", "weight")), weight_offset=float(desc.get("weight_offset", 0.0)))

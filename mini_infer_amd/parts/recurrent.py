@@ -202,3 +202,198 @@ def build_gated_delta_rule(desc: dict, dtype: torch.dtype, device, shared: dict 
         int(desc["v_head_dim"]), int(desc["taps"]), float(desc["norm_eps"]), dtype, device, names=desc.get("names"),
         suffix=str(desc.get("suffix", "")),
     )
+
+
+GLA_NAMES = {"q": "q", "k": "k", "v": "v", "gate": "g", "out": "o", "decay_down": "a1", "decay_up": "a2",
+             "decay_bias": "a2.b", "norm": "norm"}
+
+
+class GatedLinearAttention(Mixer):
+    """Linear attention whose matrix state S (head_dim x v_head_dim, float32) per head decays by a
+    gate per key channel:
+
+        q = W_q h * head_dim^-1/2,  k = W_k h,  v = W_v h
+        a = logistic(W_a2 (W_a1 h) + bias) ^ (1 / tau)                      (per head and key channel)
+        S <- diag(a_t) S + k_t v_t^T;    o_t = S^T q_t
+        y_t = W_o (rms_norm(o_t) * weight * silu(W_g h))                    (norm per head over v_head_dim)
+
+    A request's S lives in its state slot."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, decay_rank: int, tau: float,
+                 norm_eps: float, dtype: torch.dtype, device, *, names: dict[str, str] | None = None, suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        for what, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim),
+                            ("v_head_dim", v_head_dim), ("decay_rank", decay_rank)):
+            if value <= 0:
+                raise ValueError(f"gated linear attention: {what} must be positive, got {value}")
+        if tau <= 0:
+            raise ValueError(f"gated linear attention: tau must be positive, got {tau}")
+        self.hidden_size, self.num_heads, self.head_dim, self.v_head_dim = hidden_size, num_heads, head_dim, v_head_dim
+        self.decay_rank, self.tau, self.norm_eps = decay_rank, float(tau), float(norm_eps)
+        self.names = {**GLA_NAMES, **(names or {})}
+        self.suffix = suffix
+        ops.decay_state_shape(num_heads, head_dim, v_head_dim)  # (refuses widths the kernel does not take)
+        n, qk, vw = self.names, num_heads * head_dim, num_heads * v_head_dim
+        # one product yields [q | k | v | gate | decay, narrow] for every token of the step
+        self.inputs = Linear(hidden_size, [qk, qk, vw, vw, decay_rank],
+                             [n["q"], n["k"], n["v"], n["gate"], n["decay_down"]], dtype, device, suffix=suffix)
+        self.col_k, self.col_v, self.col_gate, self.col_decay = qk, 2 * qk, 2 * qk + vw, 2 * qk + 2 * vw
+        self.decay_up = Linear(decay_rank, qk, n["decay_up"], dtype, device, suffix=suffix)
+        self.out = Linear(vw, hidden_size, n["out"], dtype, device, suffix=suffix)
+        self.decay_bias: torch.Tensor | None = None
+        self.norm_weight: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        n = self.names
+        return {
+            **self.inputs.param_specs(prefix), **self.decay_up.param_specs(prefix), **self.out.param_specs(prefix),
+            prefix + n["decay_bias"]: ParamSpec((self.num_heads * self.head_dim,), dtype="float32"),
+            prefix + n["norm"]: ParamSpec((self.v_head_dim,), init="norm_weight", dtype="float32"),
+        }
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        for part in (self.inputs, self.decay_up, self.out):
+            part.load_params(prefix, get)
+        self.decay_bias = get(prefix + self.names["decay_bias"]).float().contiguous()
+        self.norm_weight = get(prefix + self.names["norm"]).float().contiguous()
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        return CacheNeeds(state=StateNeeds(ops.decay_state_shape(self.num_heads, self.head_dim, self.v_head_dim), torch.float32))
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
+        if not writes_cache:
+            raise NotImplementedError("a recurrent mixer owns its state; it cannot read another call's")
+        assert self.decay_bias is not None and self.norm_weight is not None, "gated linear attention used before its weights were loaded"
+        assert isinstance(cache.state, torch.Tensor), "gated linear attention needs its state rows from the cache manager"
+        if hasattr(x, "finish"):
+            x = x.finish()
+        proj = self.inputs.forward(x)
+        logits = self.decay_up.forward(proj[:, self.col_decay:self.col_decay + self.decay_rank])
+        readout = ops.decay_scan(
+            proj, 0, proj, self.col_k, proj, self.col_v, logits, 0, self.decay_bias, cache.state, ctx.cu_seqlens_q,
+            ctx.state_slots, heads=self.num_heads, groups=self.num_heads, dim=self.head_dim, vdim=self.v_head_dim,
+            per_head=False, inv_tau=1.0 / self.tau, q_scale=self.head_dim ** -0.5,
+        )
+        mixed = ops.readout_gate_norm(readout, proj[:, self.col_gate:], self.norm_weight, group_width=self.v_head_dim,
+                                      gate_first=False, eps=self.norm_eps)
+        return self.out.forward(mixed)
+
+
+@register_mixer("gated_linear_attention")
+def build_gated_linear_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> GatedLinearAttention:
+    return GatedLinearAttention(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["head_dim"]), int(desc["v_head_dim"]),
+        int(desc["decay_rank"]), float(desc["tau"]), float(desc["norm_eps"]), dtype, device, names=desc.get("names"),
+        suffix=str(desc.get("suffix", "")),
+    )
+
+
+SSD_NAMES = {"in": "in", "conv": "conv", "conv_bias": "conv.b", "step_bias": "dt_bias", "rate": "A_log", "skip": "D",
+             "norm": "norm", "out": "o"}
+
+
+class StateSpaceDuality(Mixer):
+    """A selective state-space layer with one decay per head (the recurrent form of state-space
+    duality).  One product yields [z | x | B | C | dt]; x, B and C pass a short causal convolution
+    with a bias and silu; then per head, with B and C shared by the heads of a group,
+
+        dt = softplus(dt + bias);   S <- exp(-exp(rate) dt) S + dt B_t x_t^T;   y_t = S^T C_t + skip * x_t
+
+    (S is state x v_head_dim, float32).  y times silu(z) is RMS-normed in `norm_groups` equal
+    parts, times a weight, and projected out.  A request's S and the last taps - 1 inputs of the
+    convolution live in its state slot."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, v_head_dim: int, state_size: int, groups: int, taps: int,
+                 norm_groups: int, norm_eps: float, dtype: torch.dtype, device, *, names: dict[str, str] | None = None,
+                 suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        for what, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("v_head_dim", v_head_dim),
+                            ("state_size", state_size), ("groups", groups), ("taps", taps), ("norm_groups", norm_groups)):
+            if value <= 0:
+                raise ValueError(f"state-space layer: {what} must be positive, got {value}")
+        self.inner = num_heads * v_head_dim
+        if num_heads % groups != 0 or self.inner % norm_groups != 0:
+            raise ValueError(f"state-space layer: heads={num_heads} must be a multiple of groups={groups}, "
+                             f"heads*v_head_dim={self.inner} of norm_groups={norm_groups}")
+        if taps > 16:
+            raise ValueError(f"state-space layer: the convolution kernel takes up to 16 taps, got {taps}")
+        self.hidden_size, self.num_heads, self.v_head_dim, self.state_size = hidden_size, num_heads, v_head_dim, state_size
+        self.groups, self.taps, self.norm_groups, self.norm_eps = groups, taps, norm_groups, float(norm_eps)
+        self.names = {**SSD_NAMES, **(names or {})}
+        ops.decay_state_shape(num_heads, state_size, v_head_dim)
+        self.channels = self.inner + 2 * groups * state_size  # what passes the convolution: x | B | C
+        n = self.names
+        self.inputs = Linear(hidden_size, 2 * self.inner + 2 * groups * state_size + num_heads, n["in"], dtype, device, suffix=suffix)
+        self.out = Linear(self.inner, hidden_size, n["out"], dtype, device, suffix=suffix)
+        self.conv_weight: torch.Tensor | None = None
+        self.conv_bias: torch.Tensor | None = None
+        self.step_bias: torch.Tensor | None = None
+        self.rate: torch.Tensor | None = None
+        self.skip: torch.Tensor | None = None
+        self.norm_weight: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        n = self.names
+        return {
+            **self.inputs.param_specs(prefix), **self.out.param_specs(prefix),
+            prefix + n["conv"]: ParamSpec((self.channels, self.taps), dtype="float32"),
+            prefix + n["conv_bias"]: ParamSpec((self.channels,), dtype="float32"),
+            prefix + n["step_bias"]: ParamSpec((self.num_heads,), dtype="float32"),
+            prefix + n["rate"]: ParamSpec((self.num_heads,), dtype="float32"),
+            prefix + n["skip"]: ParamSpec((self.num_heads,), init="norm_weight", dtype="float32"),
+            prefix + n["norm"]: ParamSpec((self.inner,), init="norm_weight", dtype="float32"),
+        }
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        n = self.names
+        self.inputs.load_params(prefix, get)
+        self.out.load_params(prefix, get)
+        self.conv_weight = get(prefix + n["conv"]).float().contiguous()
+        self.conv_bias = get(prefix + n["conv_bias"]).float().contiguous()
+        self.step_bias = get(prefix + n["step_bias"]).float().contiguous()
+        self.rate = get(prefix + n["rate"]).float().contiguous()
+        self.skip = get(prefix + n["skip"]).float().contiguous()
+        self.norm_weight = get(prefix + n["norm"]).float().contiguous()
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        state = {"recurrent": StateNeeds(ops.decay_state_shape(self.num_heads, self.state_size, self.v_head_dim), torch.float32)}
+        if self.taps > 1:
+            state["tail"] = StateNeeds((self.taps - 1, self.channels), self.dtype)
+        return CacheNeeds(state=state)
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
+        if not writes_cache:
+            raise NotImplementedError("a recurrent mixer owns its state; it cannot read another call's")
+        assert self.conv_weight is not None and self.rate is not None, "state-space layer used before its weights were loaded"
+        assert isinstance(cache.state, dict), "the state-space layer needs its state rows from the cache manager"
+        if hasattr(x, "finish"):
+            x = x.finish()
+        proj = self.inputs.forward(x)  # [z | x | B | C | dt]
+        if self.taps > 1:
+            tail = cache.state["tail"]
+        else:
+            tail = torch.empty((2, 0, self.channels), dtype=proj.dtype, device=proj.device)
+        conv = ops.short_conv(proj[:, self.inner:], self.channels, self.conv_weight, tail, ctx.cu_seqlens_q, ctx.state_slots,
+                              ctx.token_request, bias=self.conv_bias)  # [x | B | C]
+        span = self.groups * self.state_size
+        readout = ops.decay_scan(
+            conv, self.inner + span, conv, self.inner, conv, 0, proj, self.inner + self.channels, self.step_bias,
+            cache.state["recurrent"], ctx.cu_seqlens_q, ctx.state_slots, heads=self.num_heads, groups=self.groups,
+            dim=self.state_size, vdim=self.v_head_dim, per_head=True, rate=self.rate, skip=self.skip,
+        )
+        mixed = ops.readout_gate_norm(readout, proj, self.norm_weight, group_width=self.inner // self.norm_groups,
+                                      gate_first=True, eps=self.norm_eps)
+        return self.out.forward(mixed)
+
+
+@register_mixer("state_space_duality")
+def build_state_space_duality(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> StateSpaceDuality:
+    return StateSpaceDuality(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["v_head_dim"]), int(desc["state_size"]), int(desc["groups"]),
+        int(desc["taps"]), int(desc["norm_groups"]), float(desc["norm_eps"]), dtype, device, names=desc.get("names"),
+        suffix=str(desc.get("suffix", "")),
+    )
