@@ -95,7 +95,10 @@ class DecoderModel:
         return specs
 
     def optional_names(self) -> set[str]:
-        return self.head.optional_names("")
+        names = set(self.head.optional_names(""))
+        for layer, block in zip(self.spec.layers, self.blocks):
+            names |= block.optional_names(layer.prefix)
+        return names
 
     def load_params(self, get: TensorGetter) -> None:
         self.embedding.load_params("", get)

@@ -83,7 +83,7 @@ class ChunkedAttentionSizes:
     kv_heads: int
     dim: int
     vdim: int
-    chunk: int
+    chunk: int | None
     scale: float
     rot: Rotation
 
@@ -169,7 +169,8 @@ def _parse_attention(where: str, m: dict[str, Any]) -> ChunkedAttentionSizes:
     kv_heads = _positive_int(f"{where}.kv_heads", m.get("kv_heads"))
     if heads % kv_heads:
         raise ConfigError(f"{where}: heads={heads} is not a multiple of kv_heads={kv_heads}")
-    chunk = _positive_int(f"{where}.mask.size", _section(m, "mask", where).get("size"))
+    # (no mask: every earlier position is seen)
+    chunk = None if m.get("mask") is None else _positive_int(f"{where}.mask.size", _section(m, "mask", where).get("size"))
     return ChunkedAttentionSizes(
         heads=heads, kv_heads=kv_heads, dim=dim, vdim=_positive_int(f"{where}.vdim", m.get("vdim")), chunk=chunk,
         scale=_number(f"{where}.scale", m.get("scale")), rot=_parse_rotation(where, m, dim),

@@ -24,7 +24,7 @@ class ParamSpec:
     """One tensor a part reads from the checkpoint.
 
     `init` chooses the random-weights distribution: "normal" is N(0, std),
-    "norm_weight" is 1 + N(0, jitter).  `dtype` is "compute" (the engine's
+    "norm_weight" is 1 + N(0, jitter), "identity" (a matrix) I + N(0, jitter).  `dtype` is "compute" (the engine's
     dtype), "float32" (stays 32-bit whatever the engine's dtype) or "int32".
     """
 
@@ -357,6 +357,10 @@ class Block(Part):
 
     def enable_pending_output(self) -> None:
         pass
+
+    def optional_names(self, prefix: str) -> set[str]:
+        """Names a checkpoint may hold for this block without the block reading them."""
+        return set()
 
     def forward(
         self,

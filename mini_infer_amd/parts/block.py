@@ -335,8 +335,16 @@ class HyperConnectionBlock(Block):
             for sub in self._connections():
                 specs[prefix + sub + "in"] = ParamSpec((S,), init="norm_weight", dtype="float32")
                 specs[prefix + sub + "out"] = ParamSpec((S,), init="norm_weight", dtype="float32")
-                specs[prefix + sub + "mix"] = ParamSpec((S, S), init="norm_weight", dtype="float32")
+                specs[prefix + sub + "mix"] = ParamSpec((S, S), init="identity", dtype="float32")
         return specs
+
+    def optional_names(self, prefix: str) -> set[str]:
+        """A layer without a feed-forward has no use for the second sublayer's norm and vectors;
+        a checkpoint that stores them all the same is read without them."""
+        if self.feed_forward is not None:
+            return set()
+        sub = self.names["ffn_connection"]
+        return {prefix + self.names["ffn_norm"]} | {prefix + sub + what for what in ("in", "out", "mix")}
 
     def load_params(self, prefix: str, get: TensorGetter) -> None:
         for sub, part in self._children():

@@ -25,11 +25,12 @@ def default_inv_freq(rotary_dim: int, theta: float) -> torch.Tensor:
     return 1.0 / (theta**exponent)
 
 
-def exact_inv_freq(rotary_dim: int, theta: float) -> torch.Tensor:
+def exact_inv_freq(rotary_dim: int, theta: float, dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """theta^(-2j/D) evaluated in 64-bit and rounded to float32 once (`default_inv_freq` makes
-    the same table in float32 arithmetic, as the reference does, and is a last bit or two off)."""
+    the same table in float32 arithmetic, as the reference does, and is a last bit or two off).
+    `dtype=torch.float64`: not rounded yet, for a rescaling that is to be exact as well."""
     exponent = torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim
-    return torch.pow(torch.tensor(float(theta), dtype=torch.float64), -exponent).to(torch.float32)
+    return torch.pow(torch.tensor(float(theta), dtype=torch.float64), -exponent).to(dtype)
 
 
 def llama3_inv_freq(
@@ -76,7 +77,10 @@ class RotaryPosition(PositionEncoding):
         if self.rotary_dim % 2 != 0 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim={self.rotary_dim} must be even and within head_dim={head_dim}")
         self.interleaved = bool(interleaved)
-        table = (exact_inv_freq if exact_frequencies else default_inv_freq)(self.rotary_dim, float(theta))
+        if exact_frequencies:  # (the rescaling too in 64-bit; one rounding at the end)
+            table = exact_inv_freq(self.rotary_dim, float(theta), torch.float64)
+        else:
+            table = default_inv_freq(self.rotary_dim, float(theta))
         if llama3 is not None:
             table = llama3_inv_freq(
                 table,

@@ -5,7 +5,8 @@ The reference has no such mode in the library; its tests seed torch and fill
 the parameters (tests/unit/models/llama/test_llama_rope_scaling.py:79-96).  Here
 the values come from NumPy's PCG64 stream in the sorted order of tensor names,
 so any program can reproduce them from (config, seed) alone: linear and
-embedding tensors N(0, std), norm weights 1 + N(0, norm_jitter).
+embedding tensors N(0, std), norm weights 1 + N(0, norm_jitter), small square matrices
+that mix copies of a stream I + N(0, norm_jitter).
 """
 
 from __future__ import annotations
@@ -36,6 +37,8 @@ def random_tensors(
         values = rng.standard_normal(spec.shape, dtype=np.float32)
         if spec.init == "norm_weight":
             values = 1.0 + norm_jitter * values
+        elif spec.init == "identity":
+            values = np.eye(*spec.shape, dtype=np.float32) + norm_jitter * values
         elif spec.init == "normal":
             values = std * values
         else:
@@ -90,6 +93,8 @@ def fill_random_on_device(model, seed: int, *, std: float = 0.02, norm_jitter: f
         values = torch.randn(spec.shape, generator=generator, device=model.device, dtype=torch.float32)
         if spec.init == "norm_weight":
             values = 1.0 + norm_jitter * values
+        elif spec.init == "identity":
+            values = torch.eye(*spec.shape, device=model.device, dtype=torch.float32) + norm_jitter * values
         else:
             values = std * values
         return values.to(torch.float32 if spec.dtype == "float32" else model.dtype)

@@ -19,6 +19,17 @@ def _same(x):
     return x
 
 
+def bf16_round(a: np.ndarray) -> np.ndarray:
+    """What is left of `a` when it is stored in bfloat16 (round to nearest even), as float64."""
+    bits = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    bits = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) << 16
+    return bits.astype(np.uint32).view(np.float32).astype(np.float64).reshape(np.shape(a))
+
+
+def greedy(row: np.ndarray) -> int:
+    return int(np.argmax(row))
+
+
 def rms_unit(x: np.ndarray, eps: float) -> np.ndarray:
     """x divided by its root mean square over the last axis, eps inside the root."""
     return x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps)

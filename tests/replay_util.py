@@ -55,7 +55,8 @@ def oracle(cfg: dict, weights: dict, tokens, **kwargs) -> Oracle:
     )
 
 
-def assert_close(got: np.ndarray, expected, dtype: str, what: str = "") -> None:
+def assert_close(got: np.ndarray, expected, dtype: str, what: str = "", *, fp32_tol: float = FP32_TOL,
+                 bf16_max_factor: float = BF16_MAX_FACTOR) -> None:
     """`expected`: an `Oracle`, or an array (then bfloat16 falls back to a share of the largest logit)."""
     yardstick = expected if isinstance(expected, Oracle) else None
     exact = expected.exact if yardstick is not None else expected
@@ -63,9 +64,9 @@ def assert_close(got: np.ndarray, expected, dtype: str, what: str = "") -> None:
     err = np.abs(got.astype(np.float64) - exact)
     worst = np.unravel_index(np.argmax(err), err.shape)
     if dtype == "float32":
-        limit = FP32_TOL
+        limit = fp32_tol
     elif yardstick is not None:
-        limit = BF16_MAX_FACTOR * yardstick.yard_max
+        limit = bf16_max_factor * yardstick.yard_max
         if err.size >= 2000:
             p99, p99_limit = float(np.percentile(err, 99)), BF16_P99_FACTOR * yardstick.yard_p99
             assert p99 < p99_limit, f"{what} [{dtype}]: 99th percentile of the error {p99:.3e} (limit {p99_limit:.3e})"
