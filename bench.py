@@ -453,6 +453,28 @@ def zekonex_config(sizes: dict, layers: int) -> dict:
             "layers": [(delta, latent, delta, attention)[i % 4] for i in range(layers)]}
 
 
+KEMURAX_CHUNK = 8192
+KEMURAX_STREAMS = 4
+
+
+def kemurax_config(sizes: dict, layers: int) -> dict:
+    """A Kemurax model with the widths of a Llama configuration: one gated-linear-attention layer, then
+    three layers of chunked attention beside a state-space layer, and so on; every layer with a tanh-gelu
+    gated feed-forward of Llama's width; the stream in four copies.  Gated linear attention has keys half as
+    wide as the stream and values as wide, in heads of 128 x 256; the attention is Llama's (heads, key/value
+    heads, head size) with chunks of 8,192 positions; the state-space layer is as wide as the stream, heads
+    of 64 with a state of 128, one group, four taps."""
+    h, heads, kv, d = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"], sizes["head_dim"]
+    mlp = {"kind": "dense", "ff": sizes["intermediate_size"]}
+    gla = {"type": "gla", "mlp": mlp, "mixer": {"heads": max(1, h // 256), "dim": 128, "vdim": 256, "tau": 16.0}}
+    left = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": KEMURAX_CHUNK},
+            "rot": {"base": 500000.0, "dims": d, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    right = {"heads": max(1, h // 64), "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    pair = {"type": "parallel", "mlp": mlp, "mixer": {"left": left, "right": right, "left_scale": 0.5, "right_scale": 0.5}}
+    return {"architecture": "Kemurax", "vocab": sizes["vocab_size"], "width": h, "streams": KEMURAX_STREAMS, "norm": {"eps": 1e-6},
+            "layers": [gla if i % 4 == 0 else pair for i in range(layers)]}
+
+
 def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
     """What a step must move and compute, from the model's own list of tensors: bytes of every matrix
     a decode step streams (tables that are only gathered from are left out), multiply-adds of its
@@ -460,7 +482,7 @@ def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
     gathered = {"embed", "side.embed", "model.embed_tokens.weight"}
     specs = model.param_specs()
     matrix = sum(int(s.shape[0]) * int(s.shape[1]) for n, s in specs.items() if len(s.shape) == 2 and n not in gathered)
-    if "lm_head.weight" not in specs and "head" not in specs:  # a tied head streams the embedding's table
+    if "lm_head.weight" not in specs and "head" not in specs and "model.embed_tokens.weight" in specs:  # a tied head streams the embedding's table
         matrix += int(specs["model.embed_tokens.weight"].shape[0]) * int(specs["model.embed_tokens.weight"].shape[1])
     head = int(model.vocab_size) * int(model.spec.hidden_size)
     state_bytes = 0
@@ -478,6 +500,26 @@ def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
         # the recurrence: per token and head three passes over dim x vdim (decay and read, write, read out)
         attention_flops += sum(6.0 * tokens * m["heads"] * m["dim"] * m["vdim"] for t, m in mixers if t == "delta")
         # (the latent's key and value maps are applied per head to queries and outputs: counted with the matrices)
+        return {"matrix_values": matrix, "kv_values_per_request": kv_values, "state_bytes_per_request": state_bytes,
+                "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops}
+    if raw.get("architecture") == "Kemurax":
+        # attention inside chunks: a token sees the keys of its own chunk only; the recurrences keep a
+        # float32 matrix per head (read and written once a step), the state-space layer also the last
+        # inputs of its convolution; the embedding table is the head
+        matrix += head
+        chunk_of = lambda m: m["mask"]["size"]  # noqa: E731
+        lefts = [l["mixer"]["left"] for l in raw["layers"] if l["type"] == "parallel"]
+        rights = [l["mixer"]["right"] for l in raw["layers"] if l["type"] == "parallel"]
+        glas = [l["mixer"] for l in raw["layers"] if l["type"] == "gla"]
+        kv_values = sum(m["kv_heads"] * (m["dim"] + m["vdim"]) * (context % chunk_of(m) + 1) for m in lefts)
+        state_bytes = sum(2 * 4 * m["heads"] * m["dim"] * m["vdim"] for m in glas)
+        state_bytes += sum(2 * 4 * m["heads"] * m["state"] * m["vdim"] for m in rights)
+        state_bytes += sum(2 * 2 * (m["conv"] - 1) * (m["heads"] * m["vdim"] + 2 * m["groups"] * m["state"]) for m in rights)
+        pairs = lambda c: sum(i % c + 1 for i in range(tokens))  # noqa: E731
+        attention_flops = sum(2.0 * pairs(chunk_of(m)) * m["heads"] * (m["dim"] + m["vdim"]) for m in lefts)
+        # the recurrences: per token and head the decay, the outer product and the read-out over dim x vdim
+        attention_flops += sum(5.0 * tokens * m["heads"] * m["dim"] * m["vdim"] for m in glas)
+        attention_flops += sum(5.0 * tokens * m["heads"] * m["state"] * m["vdim"] for m in rights)
         return {"matrix_values": matrix, "kv_values_per_request": kv_values, "state_bytes_per_request": state_bytes,
                 "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops}
     if "layers" in raw:  # Nadosun: windowed layers
@@ -558,6 +600,8 @@ def measure_design(design: str, sizes_name: str, dtype: str, layers: int | None,
         sides = [(design, nadosun_config(sizes, layers)), ("llama", theirs)]
     elif design == "zekonex":  # beside the other design of mixed recurrent and attention layers, and beside Llama
         sides = [(design, zekonex_config(sizes, layers)), ("nadosun", nadosun_config(sizes, layers)), ("llama", theirs)]
+    elif design == "kemurax":  # beside the design whose recurrent layers also keep a matrix per head, and beside Llama
+        sides = [(design, kemurax_config(sizes, layers)), ("zekonex", zekonex_config(sizes, layers)), ("llama", theirs)]
     else:
         raise ValueError(f"no design {design!r} to compare")
     line = {"design": design, "sizes": f"{model_name} layer sizes", "layers": layers, "dtype": dtype, "window": DESIGN_WINDOW,
@@ -605,10 +649,10 @@ def main() -> int:
                         help="with --serving / --reference-workload: launch steps that have portions of prompts in them kernel "
                         "by kernel, however few their tokens (recorded steps of single tokens stay)")
     parser.add_argument(
-        "--design", default=None, choices=("nadosun", "zekonex"),
+        "--design", default=None, choices=("nadosun", "zekonex", "kemurax"),
         help="instead of the default run: prefill (one 2,048-token prompt) and decode (batch 1, --batch and 64; --steps "
         "steps, default 64 here) of that design beside Llama at the layer sizes of --sizes and equal depth "
-        "(--layers, default 12; zekonex also beside nadosun); prints one JSON line and exits",
+        "(--layers, default 12; zekonex also beside nadosun, kemurax beside zekonex); prints one JSON line and exits",
     )
     parser.add_argument("--design-alone", action="store_true", help="with --design: leave the Llama side out (for profiles)")
     parser.add_argument("--attention-batch", type=int, default=0)
