@@ -147,5 +147,37 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// V columns of a row at once: 16-byte loads of float32, 8-byte loads of bfloat16 for V = 4.
+template <typename T, int V>
+__device__ __forceinline__ void mi_load_cols(const T* p, float (&v)[V]) {
+  if constexpr (V == 1) {
+    v[0] = to_f32(p[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    const float4 got = *reinterpret_cast<const float4*>(p);
+    v[0] = got.x, v[1] = got.y, v[2] = got.z, v[3] = got.w;
+  } else {
+    const uint2 got = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(got.x << 16), v[1] = __uint_as_float(got.x & 0xFFFF0000u);
+    v[2] = __uint_as_float(got.y << 16), v[3] = __uint_as_float(got.y & 0xFFFF0000u);
+  }
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void mi_store_cols(T* p, const float (&v)[V]) {
+  if constexpr (V == 1) {
+    p[0] = from_f32<T>(v[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    union {
+      bf16_t h[4];
+      uint2 bits;
+    } packed;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) packed.h[j] = from_f32<bf16_t>(v[j]);
+    *reinterpret_cast<uint2*>(p) = packed.bits;
+  }
+}
+
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

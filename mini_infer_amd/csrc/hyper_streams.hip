@@ -48,11 +48,11 @@ __device__ __forceinline__ A block_sum_wide(A v, A* scratch) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void embed_norm_streams_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+__global__ __launch_bounds__(1024) void embed_norm_streams_kernel(const T* __restrict__ table, const int* __restrict__ ids,
                                                                  const float* __restrict__ weight, float* __restrict__ streams,
                                                                  int hidden, int vocab, int n_streams, float eps) {
   using A = typename Wide<T>::type;
-  __shared__ A scratch[4];
+  __shared__ A scratch[16];
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
@@ -73,59 +73,76 @@ __global__ __launch_bounds__(256) void embed_norm_streams_kernel(const T* __rest
   }
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void streams_update_norm_kernel(
+// S copies (a template argument: the small matrix lives in registers and its loops unroll), V
+// columns a thread at once.  A block takes a row; its threads are as many as the row has groups
+// of V columns, up to 1,024, so a step of few rows is a few loads deep.
+template <typename T, int S, int V>
+__global__ __launch_bounds__(1024) void streams_update_norm_kernel(
     const T* __restrict__ ya, int64_t a_stride, const T* __restrict__ yb, int64_t b_stride, float scale_a, float scale_b,
     const float* __restrict__ mix, const float* __restrict__ outv, const float* __restrict__ readv,
     const float* __restrict__ weight, float* __restrict__ streams, T* __restrict__ out, const int* __restrict__ rows,
-    int hidden, int n_streams, float eps) {
+    int hidden, float eps) {
   using A = typename Wide<T>::type;
-  extern __shared__ __align__(8) unsigned char lds_bytes[];
+  extern __shared__ __align__(16) unsigned char lds_bytes[];
   float* u_lds = reinterpret_cast<float*>(lds_bytes);  // [hidden]: what the norm reads
-  __shared__ A scratch[4];
-  __shared__ float mix_s[HYPER_MAX_STREAMS * HYPER_MAX_STREAMS], out_s[HYPER_MAX_STREAMS], read_s[HYPER_MAX_STREAMS];
-  const int S = n_streams;
+  __shared__ A scratch[16];
   const bool writes = mix != nullptr;
-  if (threadIdx.x < S * S) mix_s[threadIdx.x] = writes ? mix[threadIdx.x] : 0.f;
-  if (threadIdx.x < S) {
-    out_s[threadIdx.x] = writes ? outv[threadIdx.x] : 0.f;
-    read_s[threadIdx.x] = readv ? readv[threadIdx.x] : 1.f;
+  float m[S][S], ov[S], rv[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    ov[s] = writes ? outv[s] : 0.f;
+    rv[s] = readv ? readv[s] : 1.f;
+#pragma unroll
+    for (int to = 0; to < S; ++to) m[s][to] = writes ? mix[s * S + to] : 0.f;
   }
-  __syncthreads();
   const int t = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = streams + (int64_t)t * S * hidden;
   const bool store = writes && rows == nullptr;
   A ss = 0;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    float old[HYPER_MAX_STREAMS];
+  for (int c = threadIdx.x * V; c < hidden; c += blockDim.x * V) {
+    float old[S][V];
 #pragma unroll
-    for (int s = 0; s < HYPER_MAX_STREAMS; ++s)
-      if (s < S) old[s] = x[(int64_t)s * hidden + c];
-    A u = 0;
+    for (int s = 0; s < S; ++s) mi_load_cols<float, V>(x + (int64_t)s * hidden + c, old[s]);
+    float uf[V];
     if (writes) {
-      A y = 0;
-      if (ya) y = (A)scale_a * (A)to_f32(ya[(int64_t)t * a_stride + c]);
-      if (yb) y += (A)scale_b * (A)to_f32(yb[(int64_t)t * b_stride + c]);
+      float a[V], b[V];
 #pragma unroll
-      for (int to = 0; to < HYPER_MAX_STREAMS; ++to) {
-        if (to < S) {
-          A v = (A)out_s[to] * y;
+      for (int j = 0; j < V; ++j) a[j] = b[j] = 0.f;
+      if (ya) mi_load_cols<T, V>(ya + (int64_t)t * a_stride + c, a);
+      if (yb) mi_load_cols<T, V>(yb + (int64_t)t * b_stride + c, b);
+      A u[V];
 #pragma unroll
-          for (int s = 0; s < HYPER_MAX_STREAMS; ++s)
-            if (s < S) v += (A)mix_s[s * S + to] * (A)old[s];
-          const float now = (float)v;
-          if (store) x[(int64_t)to * hidden + c] = now;
-          u += (A)read_s[to] * (A)now;
+      for (int j = 0; j < V; ++j) u[j] = 0;
+#pragma unroll
+      for (int to = 0; to < S; ++to) {
+        float now[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          A y = 0;
+          if (ya) y = (A)scale_a * (A)a[j];
+          if (yb) y += (A)scale_b * (A)b[j];
+          A v = (A)ov[to] * y;
+#pragma unroll
+          for (int s = 0; s < S; ++s) v += (A)m[s][to] * (A)old[s][j];
+          now[j] = (float)v;
+          u[j] += (A)rv[to] * (A)now[j];
         }
+        if (store) mi_store_cols<float, V>(x + (int64_t)to * hidden + c, now);
       }
+#pragma unroll
+      for (int j = 0; j < V; ++j) uf[j] = (float)u[j];
     } else {
 #pragma unroll
-      for (int s = 0; s < HYPER_MAX_STREAMS; ++s)
-        if (s < S) u += (A)read_s[s] * (A)old[s];
+      for (int j = 0; j < V; ++j) {
+        A u = 0;
+#pragma unroll
+        for (int s = 0; s < S; ++s) u += (A)rv[s] * (A)old[s][j];
+        uf[j] = (float)u;
+      }
     }
-    const float uf = (float)u;
-    u_lds[c] = uf;
-    ss += (A)uf * (A)uf;
+    mi_store_cols<float, V>(u_lds + c, uf);
+#pragma unroll
+    for (int j = 0; j < V; ++j) ss += (A)uf[j] * (A)uf[j];
   }
   if (weight == nullptr) return;
   ss = block_sum_wide<A>(ss, scratch);
@@ -133,7 +150,57 @@ __global__ __launch_bounds__(256) void streams_update_norm_kernel(
   if constexpr (sizeof(T) == 4) r = 1.0 / sqrt(ss / (double)hidden + (double)eps);
   else r = 1.0f / sqrtf(ss / (float)hidden + eps);
   T* o = out + (int64_t)blockIdx.x * hidden;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = from_f32<T>((float)((A)u_lds[c] * r * (A)weight[c]));
+  for (int c = threadIdx.x * V; c < hidden; c += blockDim.x * V) {
+    float uf[V], w[V], res[V];
+    mi_load_cols<float, V>(u_lds + c, uf);
+    mi_load_cols<float, V>(weight + c, w);
+#pragma unroll
+    for (int j = 0; j < V; ++j) res[j] = (float)((A)uf[j] * r * (A)w[j]);
+    mi_store_cols<T, V>(o + c, res);
+  }
+}
+
+template <typename T, int S>
+void launch_streams(const void* ya, int64_t a_stride, const void* yb, int64_t b_stride, float scale_a, float scale_b,
+                    const float* mix, const float* outv, const float* readv, const float* weight, float* streams, void* out,
+                    const int* rows, int n_out, int hidden, float eps, hipStream_t stream) {
+  const size_t lds = (size_t)hidden * sizeof(float);
+  auto aligned = [](const void* p, size_t to) { return ((uintptr_t)p % to) == 0; };
+  const bool wide = hidden % 4 == 0 && a_stride % 4 == 0 && b_stride % 4 == 0 && aligned(ya, 4 * sizeof(T)) &&
+                    aligned(yb, 4 * sizeof(T)) && aligned(out, 4 * sizeof(T)) && aligned(streams, 16) && aligned(weight, 16);
+  if (wide) {
+    const int threads = min(1024, ceil_div(hidden / 4, MI_WAVE) * MI_WAVE);
+    streams_update_norm_kernel<T, S, 4><<<n_out, threads, lds, stream>>>((const T*)ya, a_stride, (const T*)yb, b_stride, scale_a,
+                                                                         scale_b, mix, outv, readv, weight, streams, (T*)out, rows,
+                                                                         hidden, eps);
+  } else {
+    const int threads = min(1024, ceil_div(hidden, MI_WAVE) * MI_WAVE);
+    streams_update_norm_kernel<T, S, 1><<<n_out, threads, lds, stream>>>((const T*)ya, a_stride, (const T*)yb, b_stride, scale_a,
+                                                                         scale_b, mix, outv, readv, weight, streams, (T*)out, rows,
+                                                                         hidden, eps);
+  }
+}
+
+template <typename T>
+void launch_streams_of(int n_streams, const void* ya, int64_t a_stride, const void* yb, int64_t b_stride, float scale_a,
+                       float scale_b, const float* mix, const float* outv, const float* readv, const float* weight,
+                       float* streams, void* out, const int* rows, int n_out, int hidden, float eps, hipStream_t stream) {
+#define MI_STREAMS(N)                                                                                                         \
+  case N:                                                                                                                     \
+    launch_streams<T, N>(ya, a_stride, yb, b_stride, scale_a, scale_b, mix, outv, readv, weight, streams, out, rows, n_out,  \
+                         hidden, eps, stream);                                                                                \
+    break
+  switch (n_streams) {
+    MI_STREAMS(1);
+    MI_STREAMS(2);
+    MI_STREAMS(3);
+    MI_STREAMS(4);
+    MI_STREAMS(5);
+    MI_STREAMS(6);
+    MI_STREAMS(7);
+    MI_STREAMS(8);
+  }
+#undef MI_STREAMS
 }
 
 }  // namespace
@@ -146,11 +213,12 @@ extern "C" int mi_embed_norm_streams(int dtype, const void* table, const int* id
              HYPER_MAX_STREAMS);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_norm_streams: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  const int threads = min(1024, ceil_div(hidden, MI_WAVE) * MI_WAVE);
   if (dtype == MI_F32)
-    embed_norm_streams_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)table, ids, weight, streams, hidden, vocab,
+    embed_norm_streams_kernel<float><<<num_tokens, threads, 0, stream>>>((const float*)table, ids, weight, streams, hidden, vocab,
                                                                      n_streams, eps);
   else
-    embed_norm_streams_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, weight, streams, hidden, vocab,
+    embed_norm_streams_kernel<bf16_t><<<num_tokens, threads, 0, stream>>>((const bf16_t*)table, ids, weight, streams, hidden, vocab,
                                                                       n_streams, eps);
   MI_CHECK_LAUNCH("embed_norm_streams");
   return MI_OK;
@@ -173,15 +241,12 @@ extern "C" int mi_streams_update_norm(int dtype, const void* ya, int64_t a_strid
   MI_REQUIRE((int64_t)hidden * 4 <= 60 * 1024, "streams_update_norm: hidden=%d does not fit the block's scratch", hidden);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "streams_update_norm: unknown dtype %d", dtype);
   if (n_out == 0) return MI_OK;
-  const size_t lds = (size_t)hidden * sizeof(float);
   if (dtype == MI_F32)
-    streams_update_norm_kernel<float><<<n_out, 256, lds, stream>>>((const float*)ya, a_stride, (const float*)yb, b_stride, scale_a,
-                                                                   scale_b, mix, outv, readv, weight, streams, (float*)out, rows,
-                                                                   hidden, n_streams, eps);
+    launch_streams_of<float>(n_streams, ya, a_stride, yb, b_stride, scale_a, scale_b, mix, outv, readv, weight, streams, out, rows,
+                             n_out, hidden, eps, stream);
   else
-    streams_update_norm_kernel<bf16_t><<<n_out, 256, lds, stream>>>((const bf16_t*)ya, a_stride, (const bf16_t*)yb, b_stride,
-                                                                    scale_a, scale_b, mix, outv, readv, weight, streams,
-                                                                    (bf16_t*)out, rows, hidden, n_streams, eps);
+    launch_streams_of<bf16_t>(n_streams, ya, a_stride, yb, b_stride, scale_a, scale_b, mix, outv, readv, weight, streams, out,
+                              rows, n_out, hidden, eps, stream);
   MI_CHECK_LAUNCH("streams_update_norm");
   return MI_OK;
 }
