@@ -69,7 +69,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
 enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5, EPI_GRU = 6,
-       EPI_GATED_CLAMPED = 7 };
+       EPI_GATED_CLAMPED = 7, EPI_GATED_GELU = 8 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
@@ -128,7 +128,7 @@ template <int NT, int U, int EPI, int PRO = PRO_NONE, bool LINES = false, int RT
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const FoldArgs fold) {
-  constexpr bool GATED = EPI == EPI_GATED || EPI == EPI_GATED_CLAMPED;
+  constexpr bool GATED = EPI == EPI_GATED || EPI == EPI_GATED_CLAMPED || EPI == EPI_GATED_GELU;
   constexpr bool ROPE = EPI == EPI_ROPE;
   constexpr bool ADDNORM = EPI == EPI_ADDNORM;
   constexpr bool SCALED = PRO == PRO_SCALED;
@@ -464,6 +464,13 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
           const float g = fminf((float)(bf16_t)sum[r] + fold.glu_bias[at], fold.glu_limit);
           const float u = fminf(fmaxf((float)(bf16_t)up[r] + fold.glu_bias[n + at], -fold.glu_limit), fold.glu_limit);
           sum[r] = g * mi_logistic(fold.glu_slope * g) * (u + 1.f);
+        }
+      } else if constexpr (EPI == EPI_GATED_GELU) {  // (the tanh form of gelu, as gated_mul spells it)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = (float)(bf16_t)sum[r];
+          const float f = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+          sum[r] = f * (float)(bf16_t)up[r];
         }
       } else {
 #pragma unroll
@@ -878,6 +885,13 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
                                           int64_t ldo, int m, int n, int k, hipStream_t stream) {
   const FoldArgs nothing_folded = {};
   return skinny_gated<EPI_GATED>(a, lda, w, ldw, out, ldo, m, n, k, nothing_folded, stream);
+}
+
+// out[m, n] = gelu_tanh(a . gate^T) * (a . up^T) with w = [gate; up] stacked, [2n, k].
+extern "C" int mi_gemm_skinny_geglu_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* out,
+                                         int64_t ldo, int m, int n, int k, hipStream_t stream) {
+  const FoldArgs nothing_folded = {};
+  return skinny_gated<EPI_GATED_GELU>(a, lda, w, ldw, out, ldo, m, n, k, nothing_folded, stream);
 }
 
 // out[m, n] = g * logistic(slope * g) * (u + 1), g = min(a . gate^T + bias[:n], limit), u = clamp(a . up^T +

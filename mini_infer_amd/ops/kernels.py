@@ -1598,6 +1598,36 @@ def linear_clamped_glu(x: torch.Tensor, gate_up_weight: torch.Tensor, bias: torc
     return clamped_glu(linear(x, gate_up_weight), bias, limit, slope)
 
 
+def linear_geglu(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+    """`gelu_tanh(x @ gate.T) * (x @ up.T)` with `gate_up_weight` = [gate; up] stacked, [2I, K].  bfloat16
+    with at most 32 rows runs as ONE kernel (the weight-streaming product with the activation in its
+    last step); otherwise the product and `gated_mul` run in turn.  Both round the two products to the
+    element type first and then do the same float32 arithmetic."""
+    rows, width = gate_up_weight.shape
+    if rows % 2:
+        raise KernelShapeError(f"linear_geglu: stacked weight has an odd number of rows ({rows})")
+    if (
+        x.dtype == torch.bfloat16
+        and gate_up_weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.shape[1] == width
+        and x.stride(1) == 1
+        and gate_up_weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], width, x.stride(0), gate_up_weight.stride(0), SKINNY_WIDE_MAX_ROWS)
+    ):
+        _need_cuda(x, gate_up_weight)
+        m, n = x.shape[0], rows // 2
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        library.check(
+            library.load().mi_gemm_skinny_geglu_bf16(
+                _ptr(x), x.stride(0), _ptr(gate_up_weight), gate_up_weight.stride(0), _ptr(out), out.stride(0), m, n, width, _stream(),
+            )
+        )
+        return out
+    both = linear(x, gate_up_weight)
+    return gated_mul(both[:, : rows // 2], both[:, rows // 2 :], "gelu_tanh")
+
+
 def short_conv(
     x: torch.Tensor, channels: int, taps_weight: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
     slots: torch.Tensor, token_request: torch.Tensor, bias: torch.Tensor | None = None,

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 30
+ABI_VERSION = 31
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -40,6 +40,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_gemm_skinny_attn_bf16_supported": [c_int, c_int, c_int],
     "mi_gemm_skinny_attn_bf16": [_P, _P, c_int, c_int, c_int, _P, c_int64, _P, c_int64, c_int, c_int, _P],
     "mi_gemm_skinny_swiglu_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
+    "mi_gemm_skinny_geglu_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_clamped_glu_bf16": [_P, c_int64, _P, c_int64, _P, c_float, c_float, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_rope_bf16": [
         _P, c_int64, _P, c_int64, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,

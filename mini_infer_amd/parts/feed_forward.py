@@ -60,8 +60,7 @@ class SwiGLU(FeedForward):
         else:
             if isinstance(x, ops.ScaledRows):
                 x = x.finish()
-            both = self.gate_up.forward(x)
-            act = ops.gated_mul(both[:, : self.intermediate_size], both[:, self.intermediate_size :], self.activation)
+            act = ops.linear_geglu(x, self.gate_up.weight)
         if (
             self.emit_pending_output
             and self.dtype == torch.bfloat16

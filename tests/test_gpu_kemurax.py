@@ -170,6 +170,23 @@ def test_the_gates_that_multiply_inner_rows(dtype, activation):
     np.testing.assert_allclose(got.float().cpu().numpy(), want, rtol=0, atol=tolerance(dtype, 8))
 
 
+@pytest.mark.parametrize("rows, inter, k", [(1, 24, 64), (8, 70, 256), (16, 320, 256), (17, 48, 96), (32, 130, 512), (33, 24, 64)])
+def test_gated_product_with_the_tanh_gelu_in_its_last_step(rows, inter, k):
+    """Few bfloat16 rows: one kernel, equal to the product followed by the gate's kernel up to the
+    last bit of a bfloat16 value (33 rows: the two in turn, on both sides)."""
+    from mini_infer_amd import ops
+
+    rng = np.random.default_rng(rows * inter)
+    x = dev(rng.standard_normal((rows, k)).astype(np.float32), torch.bfloat16)
+    weight = dev((rng.standard_normal((2 * inter, k)) / np.sqrt(k) * 2.5).astype(np.float32), torch.bfloat16)
+    fused = ops.linear_geglu(x, weight)
+    both = ops.linear(x, weight)
+    in_turn = ops.gated_mul(both[:, :inter], both[:, inter:], "gelu_tanh")
+    np.testing.assert_allclose(fused.float().cpu().numpy(), in_turn.float().cpu().numpy(), rtol=2 ** -7, atol=1e-6)
+    z = (x.double() @ weight.double().T).cpu().numpy()
+    np.testing.assert_allclose(fused.float().cpu().numpy(), pk.gelu_tanh(z[:, :inter]) * z[:, inter:], rtol=2 ** -6, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channels, taps", [(10, 1), (70, 2), (256, 4), (33, 7)])
 def test_the_short_convolution_with_a_bias_carries_each_requests_tail(dtype, channels, taps):
