@@ -385,14 +385,15 @@ def test_heads_normed_one_by_one_then_rotated_and_written_into_pages(dtype, head
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim, page, chunk", [
     (4, 2, 16, 24, 8, 12), (3, 3, 10, 6, 4, 5), (8, 1, 64, 64, 16, 64), (4, 1, 64, 64, 16, 50), (2, 2, 128, 128, 16, 300),
-    (4, 4, 32, 32, 32, 1), (2, 1, 64, 64, 16, 16),
+    (4, 4, 32, 32, 32, 1), (2, 1, 64, 64, 16, 16), (8, 2, 64, 64, 16, 1024), (4, 2, 16, 24, 8, 400),
 ])
 def test_attention_inside_chunks_edges_in_prompts_and_for_decoded_tokens(dtype, heads, kv_heads, dim, vdim, page, chunk):
     """One request of 333 keys in scattered pages.  Queries: a prompt's last portion of 40
     positions (it crosses chunk edges wherever chunks are shorter), and the last position alone
     as a decoded token.  For every query, head 0 is made to single out the first key of the
     query's chunk (just inside) and head 1 the key before it (just outside, with a score that
-    would take all the weight if it were seen)."""
+    would take all the weight if it were seen).  Chunks longer than the request: the first key of
+    the sequence, hundreds of positions back, is the one that stands out."""
     from mini_infer_amd import ops
 
     rng = np.random.default_rng(dim + chunk)
