@@ -186,7 +186,9 @@ class ModelRunner:
         and forgets the requests it admitted, so lengths and free pages are what they were;
         where the model keeps state of fixed size, the rows of the step's requests are copied
         aside before the forward pass and put back, so a mixer that had already updated them in
-        place leaves no trace either.
+        place leaves no trace either (a step that is replayed from a recording runs no host code
+        that can refuse, and copies nothing: with a matrix per head and layer the copy was a tenth
+        of a decode step at batch 64).
 
         `device_tokens` (int32, on the device) holds token ids the host has not read yet,
         e.g. what `sample_tokens` returned for the last step; an entry with `device_row`
@@ -255,16 +257,14 @@ class ModelRunner:
             token_ids = token_ids.astype(np.int32)
             states.flush()  # slot-table rows of requests admitted since the last step
             if self.decode_graphs is not None and self.decode_graphs.takes(index, rows, device_tokens):
-                graph, step_slots = self.decode_graphs.stage(token_ids, index, from_rows, device_tokens)
-                if states.has_state:
-                    saved = (step_slots, states.snapshot(step_slots))
+                # (a recorded step: its trial run before the recording works on the state tensors' spare
+                # row and the replay runs no host code that could refuse, so nothing is copied aside)
+                graph, _ = self.decode_graphs.stage(token_ids, index, from_rows, device_tokens)
                 logits, self.last_row_slots = graph.replay()
             elif self.decode_graphs is not None and self.decode_graphs.takes_mixed(index, [e.want for e in entries], device_tokens):
-                graph, step_slots = self.decode_graphs.stage_mixed(
+                graph, _ = self.decode_graphs.stage_mixed(
                     token_ids, index, [e.want for e in entries], from_rows, device_tokens
                 )
-                if states.has_state:
-                    saved = (step_slots, states.snapshot(step_slots))
                 logits, self.last_row_slots = graph.replay()
             else:
                 row_slots = np.fromiter(
