@@ -61,7 +61,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const int* __restrict__ token_request, const int* __restrict__ positions, T* __restrict__ out,
     int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
     int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits,
-    const float* __restrict__ slopes, int v_dim, int64_t v_row_stride, int has_sink, float sink_logit, int mask_chunk) {
+    const float* __restrict__ slopes, int v_dim, int64_t v_row_stride, int has_sink, float sink_logit, int mask_chunk,
+    float softcap, const float* __restrict__ sinks) {
   using S = typename SumType<T>::type;
   extern __shared__ __align__(8) unsigned char q_lds_bytes[];
   S* q_lds = reinterpret_cast<S*>(q_lds_bytes);  // [GT][head_dim], pre-multiplied by the scale
@@ -162,6 +163,11 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 #pragma unroll
       for (int g = 0; g < GT; ++g) {
         s_sum[g] = (s4[g][0] + s4[g][1]) + (s4[g][2] + s4[g][3]);
+        // a cap on the scaled score, softcap * tanh(score / softcap), before the distance bias
+        if (softcap > 0.f) {
+          if constexpr (sizeof(S) == 8) s_sum[g] = (S)softcap * tanh(s_sum[g] / (S)softcap);
+          else s_sum[g] = softcap * tanhf(s_sum[g] / softcap);
+        }
         s_sum[g] += (S)slope[g] * distance;
         s[g] = (float)s_sum[g];
       }
@@ -219,7 +225,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
         if (g < nh) {
           T* o = out + (int64_t)t * out_row_stride + (int64_t)(head0 + g) * v_dim + lane * VPL;
           // a sink: one more term in the denominator, exp(sink_logit) on the scores' own scale
-          const S sunk = has_sink ? (S)exp((double)sink_logit - (double)m[g]) : (S)0;
+          // (one logit for all heads, or one per query head where `sinks` is given)
+          const S sunk = has_sink ? (S)exp((double)(sinks != nullptr ? sinks[head0 + g] : sink_logit) - (double)m[g]) : (S)0;
           const S inv = (S)1 / (l[g] + sunk);
 #pragma unroll
           for (int v = 0; v < VPL; ++v)
@@ -254,7 +261,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
                                                          const float* __restrict__ part_ml,
                                                          T* __restrict__ out, int64_t out_row_stride,
                                                          int q_heads, int head_dim, int num_splits,
-                                                         int has_sink, float sink_logit) {
+                                                         int has_sink, float sink_logit, const float* __restrict__ sinks) {
   using S = typename SumType<T>::type;
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -283,7 +290,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   const float w_s = (lane < num_splits) ? expf(m_s - m_all) : 0.f;
   S l_all = 0;
   for (int s = 0; s < num_splits; ++s) l_all += (S)__shfl(l_s, s, MI_WAVE) * (S)__shfl(w_s, s, MI_WAVE);
-  if (has_sink) l_all += (S)exp((double)sink_logit - (double)m_all);
+  if (has_sink) l_all += (S)exp((double)(sinks != nullptr ? sinks[h] : sink_logit) - (double)m_all);
   const S inv = (S)1 / l_all;
   // The partial accumulators are read in batches of independent loads (a load per split
   // issued one after the other's use would cost a memory latency per split) and added in
@@ -332,7 +339,8 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
                                int num_tokens, int q_heads, int kv_heads, int head_dim,
                                int page_size, float scale, int window, int num_splits,
                                const float* slopes, hipStream_t stream, int v_dim = 0, int64_t v_row_stride = 0,
-                               int has_sink = 0, float sink_logit = 0.f, int mask_chunk = 0) {
+                               int has_sink = 0, float sink_logit = 0.f, int mask_chunk = 0, float softcap = 0.f,
+                               const float* sinks = nullptr) {
   // (values as wide as the keys and packed, no sink: what the callers that say nothing mean)
   if (v_dim <= 0) v_dim = head_dim;
   if (v_row_stride <= 0) v_row_stride = v_dim;
@@ -344,7 +352,8 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
   attn_generic_kernel<T, VPL, VEC><<<grid, MI_WAVE, lds, stream>>>(                               \
       (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
       token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
-      head_dim, page_size, scale, window, num_splits, slopes, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk)
+      head_dim, page_size, scale, window, num_splits, slopes, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk, \
+      softcap, sinks)
   if (v_dim <= 64) { if (vec) MI_ATTN_LAUNCH(1, true); else MI_ATTN_LAUNCH(1, false); }
   else if (v_dim <= 128) { if (vec) MI_ATTN_LAUNCH(2, true); else MI_ATTN_LAUNCH(2, false); }
   else if (v_dim <= 256) { if (vec) MI_ATTN_LAUNCH(4, true); else MI_ATTN_LAUNCH(4, false); }
@@ -354,7 +363,7 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
   if (num_splits > 1) {
     dim3 rgrid(num_tokens, q_heads);
     attn_reduce_kernel<T><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (T*)out, out_row_stride,
-                                                         q_heads, v_dim, num_splits, has_sink, sink_logit);
+                                                         q_heads, v_dim, num_splits, has_sink, sink_logit, sinks);
     MI_CHECK_LAUNCH("attn_reduce");
   }
   return MI_OK;
@@ -414,7 +423,8 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
 // elements that lie `v_row_stride` elements apart (a value row may be the front part of a key
 // row: pass the key pages as value pages and head_dim as the stride), key rows up to 1024 wide,
 // and optionally a sink: one more term exp(sink_logit) in the softmax's denominator that
-// carries no value, and optionally a chunked mask: a query sees only the keys of its own
+// carries no value (`sinks`, if given, holds a logit per query head instead), a cap on the scaled
+// scores (`softcap` * tanh(score / `softcap`), taken before the distance bias; 0: none), and optionally a chunked mask: a query sees only the keys of its own
 // stretch of `mask_chunk` positions (0: none).  Queries are [token][head][head_dim], outputs [token][head][v_dim];
 // part_acc holds num_tokens*q_heads*num_splits*v_dim floats.
 extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
@@ -424,7 +434,9 @@ extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, c
                                int num_tokens, int q_heads, int kv_heads, int head_dim, int v_dim,
                                int64_t v_row_stride, int page_size, int num_pages, float scale, int window,
                                int num_splits, const float* slopes, int has_sink, float sink_logit,
-                               int mask_chunk, hipStream_t stream) {
+                               int mask_chunk, float softcap, const float* sinks, hipStream_t stream) {
+  MI_REQUIRE(softcap >= 0.f, "attn_general: softcap=%g must be 0 (none) or positive", (double)softcap);
+  MI_REQUIRE(sinks == nullptr || has_sink, "attn_general: per-head sink logits come with has_sink");
   MI_REQUIRE(mask_chunk >= 0, "attn_general: mask_chunk=%d must be 0 (none) or positive", mask_chunk);
   MI_REQUIRE(v_dim > 0 && v_row_stride >= v_dim, "attn_general: value rows of %d lie %lld apart", v_dim,
              (long long)v_row_stride);
@@ -437,24 +449,26 @@ extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, c
     return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                       token_request, positions, out, out_row_stride, part_acc, part_ml,
                                       num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                      num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk);
+                                      num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk,
+                                      softcap, sinks);
   return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
-                                     num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk);
+                                     num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit, mask_chunk,
+                                      softcap, sinks);
 }
 
 // The combining step alone, for partials written by the matrix-core kernel.
 extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
                                    int64_t out_row_stride, int num_tokens, int q_heads,
                                    int head_dim, int num_splits, int has_sink, float sink_logit,
-                                   hipStream_t stream) {
+                                   const float* sinks, hipStream_t stream) {
   if (num_tokens == 0) return MI_OK;
   MI_REQUIRE(q_heads <= 65535, "attn_reduce: too many heads");
   dim3 rgrid(num_tokens, q_heads);
   attn_reduce_kernel<bf16_t><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (bf16_t*)out,
                                                             out_row_stride, q_heads, head_dim,
-                                                            num_splits, has_sink, sink_logit);
+                                                            num_splits, has_sink, sink_logit, sinks);
   MI_CHECK_LAUNCH("attn_reduce");
   return MI_OK;
 }

@@ -70,7 +70,8 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     bf16_t* __restrict__ out, int64_t out_row_stride, float* __restrict__ part_acc,
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
     int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request,
-    int pair_group, int first_token, int has_sink, float sink_log2, int mask_chunk) {
+    int pair_group, int first_token, int has_sink, float sink_log2, int mask_chunk,
+    const float* __restrict__ sinks) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   // PS != 0: the page size is this constant (divisions become shifts, value offsets
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
@@ -725,7 +726,9 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     }
     if (num_splits == 1) {
       // a sink: one more term in the denominator (its score, like all others here, in log2 units)
-      const float inv = 1.f / (l_run[rg] + (has_sink ? exp2f(sink_log2 - m_run[rg]) : 0.f));
+      // (one logit for all heads, or one per query head where `sinks` is given)
+      const float sunk_log2 = sinks != nullptr ? sinks[head[rg]] * LOG2E : sink_log2;
+      const float inv = 1.f / (l_run[rg] + (has_sink ? exp2f(sunk_log2 - m_run[rg]) : 0.f));
       bf16_t* o = out + (int64_t)token[rg] * out_row_stride + (int64_t)head[rg] * D + quad * 4;
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db) {
@@ -752,7 +755,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
 extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
                                    int64_t out_row_stride, int num_tokens, int q_heads,
                                    int head_dim, int num_splits, int has_sink, float sink_logit,
-                                   hipStream_t stream);
+                                   const float* sinks, hipStream_t stream);
 
 static int heads_per_block_for(int group, int rows) { return group < rows ? group : rows; }
 
@@ -810,7 +813,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             int head_dim, int page_size, int num_pages, float scale, int window,
                             int num_splits, int shape, int one_tile_per_request,
                             int first_token, int combine, int has_sink, float sink_logit, int mask_chunk,
-                            hipStream_t stream) {
+                            const float* sinks, hipStream_t stream) {
+  MI_REQUIRE(sinks == nullptr || has_sink, "attn_mfma: per-head sink logits come with has_sink");
   MI_REQUIRE(mask_chunk >= 0, "attn_mfma: mask_chunk=%d must be 0 (none) or positive", mask_chunk);
   MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
@@ -870,7 +874,8 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       block_table, max_blocks, cu_seqlens_q, positions, num_requests, (bf16_t*)out,               \
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
-      num_splits, hb, tq, one_tile_per_request, pair_group, first_token, has_sink, sink_logit * LOG2E, mask_chunk)
+      num_splits, hb, tq, one_tile_per_request, pair_group, first_token, has_sink, sink_logit * LOG2E, mask_chunk, \
+      sinks)
 // (head sizes above 128 have no wide shape and were refused above: their cases name the 128 kernel,
 // so that nothing is compiled for them)
 #define MI_LAUNCH_P(DD, PP)                                                                       \
@@ -899,7 +904,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
     const int64_t first_slot = (int64_t)first_token * q_heads * num_splits;
     return mi_attn_reduce_bf16(part_acc + first_slot * head_dim, part_ml + first_slot * 2,
                                (bf16_t*)out + (int64_t)first_token * out_row_stride, out_row_stride,
-                               num_tokens, q_heads, head_dim, num_splits, has_sink, sink_logit, stream);
+                               num_tokens, q_heads, head_dim, num_splits, has_sink, sink_logit, sinks, stream);
   }
   return MI_OK;
 }

@@ -23,7 +23,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_col, int q_head_width, int q_rot_at, int c_col,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, const float* __restrict__ norm_weight,
     const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ queries, int64_t queries_stride,
-    T* __restrict__ latent_out, int heads, int rank, int rot, float eps) {
+    T* __restrict__ latent_out, int heads, int rank, int rot, float eps, const T* __restrict__ down,
+    int64_t down_stride) {
   __shared__ float scratch[4];
   __shared__ double scratch_wide[4];
   constexpr bool WIDE = sizeof(T) == 4;
@@ -57,7 +58,8 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
 
   const int slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
   if (slot < 0 && latent_out == nullptr) return;  // (the whole block leaves together)
-  const T* x = row + c_col;
+  // ([x_c | x_r] lie in `proj`'s rows, or in rows of their own where the queries come from a product of their own)
+  const T* x = (down != nullptr ? down + (int64_t)t * down_stride : row) + c_col;
   float squares = 0.f;
   double squares_wide = 0.0;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(256) void latent_expand_kernel(
     const T* __restrict__ proj, int64_t proj_stride, int q_head_width, int q_rot_at, int r_col,
     const T* __restrict__ k_up, int64_t k_up_stride, const T* __restrict__ v_up, int64_t v_up_stride,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, T* __restrict__ qkv, int64_t qkv_stride, int heads,
-    int dim, int rot, int vdim) {
+    int dim, int rot, int vdim, const T* __restrict__ down, int64_t down_stride) {
   const int t = blockIdx.x;
   const int half = rot / 2, D = dim + rot;
   const T* row = proj + (int64_t)t * proj_stride;
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(256) void latent_expand_kernel(
     } else {
       const int i = (d - dim) / 2, odd = (d - dim) & 1;
       const T* qx = row + h * q_head_width + q_rot_at + 2 * i;
-      const T* kx = row + r_col + 2 * i;
+      const T* kx = (down != nullptr ? down + (int64_t)t * down_stride : row) + r_col + 2 * i;
       const float q0 = to_f32(qx[0]), q1 = to_f32(qx[1]), k0 = to_f32(kx[0]), k1 = to_f32(kx[1]);
       qv = from_f32<T>(odd ? q1 * c[i] + q0 * s[i] : q0 * c[i] - q1 * s[i]);
       kv = from_f32<T>(odd ? k1 * c[i] + k0 * s[i] : k0 * c[i] - k1 * s[i]);
@@ -141,11 +143,12 @@ __global__ __launch_bounds__(256) void latent_expand_kernel(
 extern "C" int mi_latent_expand(int dtype, const void* proj, int64_t proj_stride, int q_head_width, int q_rot_at, int r_col,
                                 const void* k_up, int64_t k_up_stride, const void* v_up, int64_t v_up_stride,
                                 const float* cos_t, const float* sin_t, void* qkv, int64_t qkv_stride, int num_tokens,
-                                int heads, int dim, int rot, int vdim, hipStream_t stream) {
+                                int heads, int dim, int rot, int vdim, const void* down, int64_t down_stride,
+                                hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && heads > 0 && dim > 0 && rot >= 0 && rot % 2 == 0 && vdim > 0 && vdim <= dim + rot,
              "latent_expand: bad sizes tokens=%d heads=%d dim=%d rot=%d vdim=%d", num_tokens, heads, dim, rot, vdim);
   MI_REQUIRE(q_rot_at == dim && q_head_width >= dim + rot, "latent_expand: a query head is [plain (dim) | to rotate (rot)]");
-  MI_REQUIRE(proj_stride >= (int64_t)heads * q_head_width && proj_stride >= r_col + (int64_t)rot && r_col >= 0 &&
+  MI_REQUIRE(proj_stride >= (int64_t)heads * q_head_width && (down != nullptr ? down_stride : proj_stride) >= r_col + (int64_t)rot && r_col >= 0 &&
                  k_up_stride >= (int64_t)heads * dim && v_up_stride >= (int64_t)heads * vdim &&
                  qkv_stride >= 3 * (int64_t)heads * (dim + rot),
              "latent_expand: row strides shorter than a row");
@@ -154,11 +157,12 @@ extern "C" int mi_latent_expand(int dtype, const void* proj, int64_t proj_stride
   if (dtype == MI_F32)
     latent_expand_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (const float*)proj, proj_stride, q_head_width, q_rot_at, r_col, (const float*)k_up, k_up_stride, (const float*)v_up,
-        v_up_stride, cos_t, sin_t, (float*)qkv, qkv_stride, heads, dim, rot, vdim);
+        v_up_stride, cos_t, sin_t, (float*)qkv, qkv_stride, heads, dim, rot, vdim, (const float*)down, down_stride);
   else
     latent_expand_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (const bf16_t*)proj, proj_stride, q_head_width, q_rot_at, r_col, (const bf16_t*)k_up, k_up_stride,
-        (const bf16_t*)v_up, v_up_stride, cos_t, sin_t, (bf16_t*)qkv, qkv_stride, heads, dim, rot, vdim);
+        (const bf16_t*)v_up, v_up_stride, cos_t, sin_t, (bf16_t*)qkv, qkv_stride, heads, dim, rot, vdim, (const bf16_t*)down,
+        down_stride);
   MI_CHECK_LAUNCH("latent_expand");
   return MI_OK;
 }
@@ -168,17 +172,18 @@ extern "C" int mi_latent_expand(int dtype, const void* proj, int64_t proj_stride
 // x_r (rot)].  k_pages: [num_pages * page_size][rank + rot] (one key head); slot_mapping may be
 // null (nothing is written: a call that reads another's pages).  queries: [tokens, heads * (rank
 // + rot)] (row stride) or null; only the last rot columns of every head are written here.
-// latent_out: [tokens, rank] or null, a copy of the normed latents.
+// latent_out: [tokens, rank] or null, a copy of the normed latents.  down (may be null): rows of their own
+// that hold [x_c | x_r] from c_col on, where the queries come from a product of their own.
 extern "C" int mi_latent_prepare(int dtype, const void* proj, int64_t proj_stride, int q_col, int q_head_width,
                                  int q_rot_at, int c_col, const float* cos_t, const float* sin_t,
                                  const float* norm_weight, const int* slot_mapping, void* k_pages, void* queries,
                                  int64_t queries_stride, void* latent_out, int num_tokens, int heads, int rank, int rot,
-                                 float eps, hipStream_t stream) {
+                                 float eps, const void* down, int64_t down_stride, hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && heads > 0 && rank > 0 && rot >= 0 && rot % 2 == 0,
              "latent_prepare: bad sizes tokens=%d heads=%d rank=%d rot=%d", num_tokens, heads, rank, rot);
   MI_REQUIRE(q_rot_at >= 0 && q_rot_at + rot <= q_head_width, "latent_prepare: the rotated part lies outside a query head");
   MI_REQUIRE(q_col >= 0 && c_col >= 0 && proj_stride >= q_col + (int64_t)heads * q_head_width &&
-                 proj_stride >= c_col + (int64_t)rank + rot,
+                 (down != nullptr ? down_stride : proj_stride) >= c_col + (int64_t)rank + rot,
              "latent_prepare: columns outside a row of the projections");
   MI_REQUIRE(queries == nullptr || queries_stride >= (int64_t)heads * (rank + rot),
              "latent_prepare: query rows shorter than heads * (rank + rot)");
@@ -189,11 +194,12 @@ extern "C" int mi_latent_prepare(int dtype, const void* proj, int64_t proj_strid
   if (dtype == MI_F32)
     latent_prepare_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (const float*)proj, proj_stride, q_col, q_head_width, q_rot_at, c_col, cos_t, sin_t, norm_weight, slot_mapping,
-        (float*)k_pages, (float*)queries, queries_stride, (float*)latent_out, heads, rank, rot, eps);
+        (float*)k_pages, (float*)queries, queries_stride, (float*)latent_out, heads, rank, rot, eps, (const float*)down, down_stride);
   else
     latent_prepare_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (const bf16_t*)proj, proj_stride, q_col, q_head_width, q_rot_at, c_col, cos_t, sin_t, norm_weight, slot_mapping,
-        (bf16_t*)k_pages, (bf16_t*)queries, queries_stride, (bf16_t*)latent_out, heads, rank, rot, eps);
+        (bf16_t*)k_pages, (bf16_t*)queries, queries_stride, (bf16_t*)latent_out, heads, rank, rot, eps, (const bf16_t*)down,
+        down_stride);
   MI_CHECK_LAUNCH("latent_prepare");
   return MI_OK;
 }

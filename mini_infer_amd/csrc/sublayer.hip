@@ -692,6 +692,122 @@ extern "C" int mi_qk_norm_kv_write(int dtype, void* qk, int64_t row_stride, cons
 }
 
 // ---------------------------------------------------------------------------
+// The same with values of their own: row layout [q: q_width | k: kv_heads * head_dim | v: kv_heads * v_dim].
+//   q <- q * rsqrt(mean(q^2) + eps) * qw      (in place)
+//   key page slot   <- k * rsqrt(mean(k^2) + eps) * kw
+//   value page slot <- v, or (1 - mix) * v + mix * other[t] where another layer's values of the
+//                      same tokens are given (`other` [tokens, kv_heads * v_dim], `mix` one float32)
+// kv_heads = 0 or no slots: q only.
+// ---------------------------------------------------------------------------
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void qkv_norm_write_kernel(
+    T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ qw, const float* __restrict__ kw,
+    const T* __restrict__ other, int64_t other_stride, const float* __restrict__ mix,
+    const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int q_width,
+    int kv_heads, int head_dim, int v_dim, int page_size, int v_transposed, float eps) {
+  using A = typename Wide<T>::type;
+  __shared__ A scratch[16];
+  const int t = blockIdx.x;
+  T* row = qkv + (int64_t)t * row_stride;
+  const int k_width = kv_heads * head_dim, v_width = kv_heads * v_dim;
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;
+  A q_squares = 0, k_squares = 0;
+  for (int i = first; i < q_width; i += stride) {
+    float v[VEC];
+    load_cols<T, VEC>(row + i, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) q_squares += (A)v[j] * (A)v[j];
+  }
+  for (int i = first; i < k_width; i += stride) {
+    float v[VEC];
+    load_cols<T, VEC>(row + q_width + i, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) k_squares += (A)v[j] * (A)v[j];
+  }
+  const A q_inv = inv_root(block_total<A>(q_squares, scratch) / (A)q_width, (A)eps);
+  const bool writes = k_width > 0 && slot_mapping != nullptr;
+  const A k_inv = writes ? inv_root(block_total<A>(k_squares, scratch) / (A)k_width, (A)eps) : (A)0;
+  for (int i = first; i < q_width; i += stride) {
+    float v[VEC], w[VEC];
+    load_cols<T, VEC>(row + i, v);
+    load_cols<float, VEC>(qw + i, w);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) v[j] = (float)(((A)v[j] * q_inv) * (A)w[j]);
+    store_cols<T, VEC>(row + i, v);
+  }
+  if (!writes) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size;
+  for (int e = first; e < k_width; e += stride) {
+    const int h = e / head_dim, d = e % head_dim;  // (VEC divides head_dim: the VEC values lie in one head)
+    float raw[VEC], w[VEC];
+    load_cols<T, VEC>(row + q_width + e, raw);
+    load_cols<float, VEC>(kw + e, w);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) raw[j] = (float)(((A)raw[j] * k_inv) * (A)w[j]);
+    store_cols<T, VEC>(k_pages + (((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d, raw);
+  }
+  const A lam = (other != nullptr) ? (A)mix[0] : (A)0;
+  for (int e = first; e < v_width; e += stride) {
+    const int h = e / v_dim, d = e % v_dim;  // (VEC divides v_dim)
+    float val[VEC];
+    load_cols<T, VEC>(row + q_width + k_width + e, val);
+    if (other != nullptr) {
+      float first_val[VEC];
+      load_cols<T, VEC>(other + (int64_t)t * other_stride + e, first_val);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) val[j] = (float)(((A)1 - lam) * (A)val[j] + lam * (A)first_val[j]);
+    }
+    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * v_dim;
+    if (v_transposed) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v_pages[chunk + (int64_t)(d + j) * page_size + off] = from_f32<T>(val[j]);
+    } else {
+      store_cols<T, VEC>(v_pages + chunk + (int64_t)off * v_dim + d, val);
+    }
+  }
+}
+
+extern "C" int mi_qkv_norm_write(int dtype, void* qkv, int64_t row_stride, const float* qw, const float* kw,
+                                 const void* other, int64_t other_stride, const float* mix, const int* slot_mapping,
+                                 void* k_pages, void* v_pages, int num_tokens, int q_width, int kv_heads, int head_dim,
+                                 int v_dim, int page_size, int num_pages, int v_transposed, float eps,
+                                 hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && q_width > 0 && kv_heads >= 0 && head_dim > 0 && v_dim > 0,
+             "qkv_norm_write: bad sizes tokens=%d q_width=%d kv_heads=%d head_dim=%d v_dim=%d", num_tokens, q_width, kv_heads,
+             head_dim, v_dim);
+  MI_REQUIRE(row_stride >= (int64_t)q_width + (int64_t)kv_heads * (head_dim + v_dim),
+             "qkv_norm_write: row stride %lld is shorter than q, k and v together", (long long)row_stride);
+  MI_REQUIRE(kv_heads == 0 || slot_mapping == nullptr || (page_size > 0 && num_pages > 0 && k_pages && v_pages && kw),
+             "qkv_norm_write: pages and the key norm's weight are needed to write keys and values");
+  MI_REQUIRE(other == nullptr || (mix != nullptr && other_stride >= (int64_t)kv_heads * v_dim),
+             "qkv_norm_write: values to mix in come with their weight and rows at least as wide as the values");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "qkv_norm_write: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  const int64_t step = dtype == MI_F32 ? 4 : 8;
+  const bool vec = q_width % step == 0 && head_dim % step == 0 && v_dim % step == 0 && row_stride % step == 0 &&
+                   other_stride % step == 0 && aligned16(qkv) && aligned16(qw) && aligned16(kw) && aligned16(other) &&
+                   aligned16(k_pages) && aligned16(v_pages);
+  const int threads = row_block(num_tokens, (q_width + kv_heads * (head_dim + v_dim)) / (vec ? 4 : 1));
+#define MI_QKV(T, VEC)                                                                                              \
+  qkv_norm_write_kernel<T, VEC><<<num_tokens, threads, 0, stream>>>(                                                \
+      (T*)qkv, row_stride, qw, kw, (const T*)other, other_stride, mix, slot_mapping, (T*)k_pages, (T*)v_pages,      \
+      q_width, kv_heads, head_dim, v_dim, page_size, v_transposed, eps)
+  if (dtype == MI_F32) {
+    if (vec) MI_QKV(float, 4);
+    else MI_QKV(float, 1);
+  } else {
+    if (vec) MI_QKV(bf16_t, 4);
+    else MI_QKV(bf16_t, 1);
+  }
+#undef MI_QKV
+  MI_CHECK_LAUNCH("qkv_norm_write");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
 // PolyNorm over a token's feed-forward values z [width]:
 //   out = a * z / rms(z) + b * z^2 / rms(z^2) + c * z^3 / rms(z^3) + e,   rms(v) = sqrt(mean(v^2) + eps)
 // `coef` = (a, b, c, e) float32.  One block a row.

@@ -1,6 +1,6 @@
 """Model assembly.  Importing this package registers the built-in architecture."""
 
-from mini_infer_amd.models import kemurax, llama, nadosun, zekonex  # noqa: F401
+from mini_infer_amd.models import kemurax, kunudra, llama, nadosun, zekonex  # noqa: F401
 from mini_infer_amd.models.decoder import DecoderModel
 from mini_infer_amd.models.spec import Architecture, LayerCall, LayerSpec, ModelSpec
 from mini_infer_amd.registry import ARCHITECTURES

@@ -112,17 +112,28 @@ class DecoderModel:
     # -- cache ----------------------------------------------------------------
 
     def cache_needs(self, page_size: int) -> list[CacheNeeds | None]:
-        """Per call in `order`: what its own cache must hold, or None if it reads another's."""
-        return [
+        """Per call in `order`: what its own cache must hold, or None if it reads another's; then,
+        if the embedding keeps state, its needs."""
+        needs = [
             None if call.reads_cache_of is not None else self.blocks[call.layer].mixer.cache_needs(page_size)
             for call in self.spec.order
         ]
+        # an embedding that keeps state of its own gets one more cache, behind the calls'
+        own = self.embedding.cache_needs(page_size) if hasattr(self.embedding, "cache_needs") else None
+        if own is not None:
+            if own.pages is not None:
+                raise ValueError("an embedding keeps state of fixed size only, no pages")
+            needs.append(own)
+        return needs
 
     # -- forward --------------------------------------------------------------
 
     def forward(self, ctx: StepContext, caches: list[LayerCache]) -> torch.Tensor:
         """Logits [len(ctx.logit_rows), vocab] float32.  `caches[i]` belongs to call i."""
-        residual = self.embedding.forward(ctx)
+        if len(caches) > len(self.spec.order):  # (the embedding's own state rows)
+            residual = self.embedding.forward(ctx, caches[len(self.spec.order)])
+        else:
+            residual = self.embedding.forward(ctx)
         delta: torch.Tensor | None = None
         for i, call in enumerate(self.spec.order):
             own = call.reads_cache_of is None

@@ -912,6 +912,8 @@ def paged_attention(
     v_head_dim: int | None = None,
     sink_logit: float | None = None,
     chunk: int | None = None,
+    sinks: torch.Tensor | None = None,
+    softcap: float | None = None,
 ) -> torch.Tensor | AttentionPieces:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
 
@@ -920,6 +922,10 @@ def paged_attention(
     of its key row.  `sink_logit`: the softmax's denominator gets one more term
     exp(sink_logit), a sink that carries no value (both attention kernels know it; uncombined
     `AttentionPieces` do not).  Values of a width of their own run the plain kernel.
+
+    `sinks` (float32 [q_heads], optional): a sink logit per query head instead of one for all
+    (both kernels).  `softcap`: every scaled score becomes `softcap * tanh(score / softcap)` before
+    slopes are applied; only the plain kernel knows it.
 
     `chunk`: a chunked mask: the token at position p sees only keys from `p // chunk * chunk` on
     (its own stretch of `chunk` positions, counted from the sequence's start); it combines with
@@ -945,14 +951,22 @@ def paged_attention(
     """
     if chunk is not None and chunk <= 0:
         raise KernelShapeError(f"a chunked mask needs a positive chunk, got {chunk}")
-    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or (
-        (sink_logit is not None or chunk is not None) and not v_transposed
+    if sinks is not None:
+        _need_cuda(sinks)
+        _need_contiguous("sinks", sinks)
+        if sinks.dtype != torch.float32 or sinks.numel() != q_heads:
+            raise KernelShapeError(f"sinks must be float32 [{q_heads}], got {sinks.dtype} x {sinks.numel()}")
+        if sink_logit is not None:
+            raise KernelShapeError("a sink logit for all heads or one per head, not both")
+    has_sink = sink_logit is not None or sinks is not None
+    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or softcap is not None or (
+        (has_sink or chunk is not None) and not v_transposed
     ):
         return _paged_attention_general(
             q, k_pages, v_pages, block_table, token_request, positions, q_heads=q_heads, kv_heads=kv_heads,
             head_dim=head_dim, v_head_dim=head_dim if v_head_dim is None else int(v_head_dim), scale=scale,
             window=window, max_seq_len=max_seq_len, v_transposed=v_transposed, slopes=slopes, sink_logit=sink_logit,
-            chunk=chunk,
+            chunk=chunk, sinks=sinks, softcap=softcap,
         )
     _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, cu_seqlens_q)
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
@@ -1027,8 +1041,8 @@ def paged_attention(
                 _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
                 _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens, num_tiles, _ptr(out), out.stride(0),
                 _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads, head_dim, page_size, num_pages, float(scale),
-                int(window or 0), splits, shape, 0, 0, 1, int(sink_logit is not None), float(sink_logit or 0.0),
-                int(chunk or 0), _stream(),
+                int(window or 0), splits, shape, 0, 0, 1, int(has_sink), float(sink_logit or 0.0),
+                int(chunk or 0), _ptr(sinks), _stream(),
             )
         )
         return out
@@ -1071,8 +1085,8 @@ def paged_attention(
                     num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
                     shape, int(one_tile_per_request), first_token,
-                    0 if (leave_pieces and splits > 1) else 1, int(sink_logit is not None), float(sink_logit or 0.0),
-                    int(chunk or 0), _stream(),
+                    0 if (leave_pieces and splits > 1) else 1, int(has_sink), float(sink_logit or 0.0),
+                    int(chunk or 0), _ptr(sinks), _stream(),
                 )
             )
             if leave_pieces and splits > 1:
@@ -1090,7 +1104,7 @@ def paged_attention(
             run(0, leading_single)
             run(leading_single, num_requests)
         else:
-            pieces = run(0, num_requests, leave_pieces=not combine and sink_logit is None and chunk is None
+            pieces = run(0, num_requests, leave_pieces=not combine and not has_sink and chunk is None
                          and leading_single == num_requests)
             if pieces is not None:
                 return pieces
@@ -1119,9 +1133,12 @@ def _paged_attention_general(
     token_request: torch.Tensor, positions: torch.Tensor, *, q_heads: int, kv_heads: int, head_dim: int,
     v_head_dim: int, scale: float, window: int | None, max_seq_len: int, v_transposed: bool,
     slopes: torch.Tensor | None, sink_logit: float | None, chunk: int | None = None,
+    sinks: torch.Tensor | None = None, softcap: float | None = None,
 ) -> torch.Tensor:
     """The plain attention kernel with everything it can be told: see `paged_attention`."""
-    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, slopes)
+    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, slopes, sinks)
+    if softcap is not None and not softcap > 0:
+        raise KernelShapeError(f"a cap on the scores must be positive, got {softcap}")
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
                     ("token_request", token_request), ("positions", positions), ("slopes", slopes)):
         _need_contiguous(name, t)
@@ -1169,7 +1186,8 @@ def _paged_attention_general(
             _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(values), _ptr(block_table), block_table.shape[1],
             _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), tokens,
             q_heads, kv_heads, head_dim, v_head_dim, v_row_stride, page_size, num_pages, float(scale), int(window or 0),
-            splits, _ptr(slopes), int(sink_logit is not None), float(sink_logit or 0.0), int(chunk or 0), _stream(),
+            splits, _ptr(slopes), int(sink_logit is not None or sinks is not None), float(sink_logit or 0.0), int(chunk or 0),
+            float(softcap or 0.0), _ptr(sinks), _stream(),
         )
     )
     return out
@@ -1724,7 +1742,7 @@ def gated_delta(
 def latent_prepare(
     proj: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor, slot_mapping: torch.Tensor | None,
     k_pages: torch.Tensor | None, queries: torch.Tensor | None, *, heads: int, q_head_width: int, q_rot_at: int, c_col: int,
-    rank: int, rot: int, eps: float, latent_out: torch.Tensor | None = None,
+    rank: int, rot: int, eps: float, latent_out: torch.Tensor | None = None, down: torch.Tensor | None = None,
 ) -> None:
     """What a latent attention layer does between its projections and its attention.  `proj`
     [T, ...] holds the query heads (`q_head_width` columns each from column 0 on, the part to
@@ -1732,8 +1750,13 @@ def latent_prepare(
     Writes `[rms_norm(x_c) * norm_weight | rotated x_r]` into the token's slot of `k_pages`
     ([num_pages, 1, page_size, rank + rot]; nothing with `slot_mapping=None`) and each head's
     rotated query part into the last `rot` columns of its [rank + rot] wide piece of `queries`
-    (`queries=None`: not wanted).  `latent_out` [T, rank]: a copy of the normed latents, if wanted."""
-    _need_cuda(proj, cos, sin, norm_weight, slot_mapping, k_pages, queries, latent_out)
+    (`queries=None`: not wanted).  `latent_out` [T, rank]: a copy of the normed latents, if wanted.
+    `down` [T, ...]: rows of their own that hold [x_c | x_r] from `c_col` on, where the queries come
+    from a product of their own (`proj` then holds the query heads alone)."""
+    _need_cuda(proj, cos, sin, norm_weight, slot_mapping, k_pages, queries, latent_out, down)
+    if down is not None and (down.dim() != 2 or down.stride(1) != 1 or down.dtype != proj.dtype or down.shape[0] != proj.shape[0]
+                             or down.shape[1] < c_col + rank + rot):
+        raise KernelShapeError(f"latent_prepare: the latent rows must be {proj.dtype} [{proj.shape[0]}, >= {c_col + rank + rot}]")
     _need_contiguous("latent_out", latent_out)
     if latent_out is not None and (latent_out.dtype != proj.dtype or tuple(latent_out.shape) != (proj.shape[0], rank)):
         raise KernelShapeError(f"latent_prepare: latent_out is {proj.dtype} [{proj.shape[0]}, {rank}], got {latent_out.dtype} {tuple(latent_out.shape)}")
@@ -1742,7 +1765,7 @@ def latent_prepare(
     _need_int32("slot_mapping", slot_mapping)
     _need_f32("norm_weight", norm_weight)
     tokens = proj.shape[0]
-    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < max(heads * q_head_width, c_col + rank + rot):
+    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < max(heads * q_head_width, 0 if down is not None else c_col + rank + rot):
         raise KernelShapeError(f"latent_prepare: the projections' rows are too short, got {tuple(proj.shape)}")
     if queries is not None and (queries.dtype != proj.dtype or queries.dim() != 2 or queries.stride(1) != 1
                                 or tuple(queries.shape) != (tokens, heads * (rank + rot))):
@@ -1760,14 +1783,15 @@ def latent_prepare(
         library.load().mi_latent_prepare(
             _dtype_code(proj), _ptr(proj), proj.stride(0), 0, int(q_head_width), int(q_rot_at), int(c_col), _ptr(cos), _ptr(sin),
             _ptr(norm_weight), _ptr(slot_mapping), _ptr(k_pages) if slot_mapping is not None else None, _ptr(queries),
-            0 if queries is None else queries.stride(0), _ptr(latent_out), tokens, heads, rank, rot, float(eps), _stream(),
+            0 if queries is None else queries.stride(0), _ptr(latent_out), tokens, heads, rank, rot, float(eps),
+            _ptr(down), 0 if down is None else down.stride(0), _stream(),
         )
     )
 
 
 def latent_expand(
     proj: torch.Tensor, k_up: torch.Tensor, v_up: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, heads: int,
-    dim: int, rot: int, vdim: int, r_col: int,
+    dim: int, rot: int, vdim: int, r_col: int, down: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """One row [q | k | v] per token with `heads` heads of D = dim + rot columns each, from a latent
     attention layer's projections (`proj`: query heads [plain (dim) | to rotate (rot)] from column 0
@@ -1782,13 +1806,18 @@ def latent_expand(
     tokens, width = proj.shape[0], dim + rot
     if cos.dtype != torch.float32 or tuple(cos.shape) != (tokens, rot // 2) or sin.shape != cos.shape or sin.dtype != torch.float32:
         raise KernelShapeError(f"latent_expand: cos/sin must be float32 [{tokens}, {rot // 2}]")
-    if k_up.shape[1] != heads * dim or v_up.shape[1] != heads * vdim or vdim > width or proj.shape[1] < max(heads * width, r_col + rot):
+    if down is not None and (down.dim() != 2 or down.stride(1) != 1 or down.dtype != proj.dtype or down.shape[0] != tokens
+                             or down.shape[1] < r_col + rot):
+        raise KernelShapeError("latent_expand: the rows that hold the shared part do not fit")
+    if k_up.shape[1] != heads * dim or v_up.shape[1] != heads * vdim or vdim > width or proj.shape[1] < max(
+            heads * width, 0 if down is not None else r_col + rot):
         raise KernelShapeError("latent_expand: the projections do not hold what the sizes say")
     qkv = torch.empty((tokens, 3 * heads * width), dtype=proj.dtype, device=proj.device)
     library.check(
         library.load().mi_latent_expand(
             _dtype_code(proj), _ptr(proj), proj.stride(0), width, dim, int(r_col), _ptr(k_up), k_up.stride(0), _ptr(v_up),
-            v_up.stride(0), _ptr(cos), _ptr(sin), _ptr(qkv), qkv.stride(0), tokens, heads, dim, rot, vdim, _stream(),
+            v_up.stride(0), _ptr(cos), _ptr(sin), _ptr(qkv), qkv.stride(0), tokens, heads, dim, rot, vdim,
+            _ptr(down), 0 if down is None else down.stride(0), _stream(),
         )
     )
     return qkv
@@ -2154,3 +2183,269 @@ class WeightedSum:
 
     def finish(self) -> torch.Tensor:
         return (self.scale_a * self.a.float() + self.scale_b * self.b.float()).to(self.a.dtype)
+
+
+# ----------------------------------------------------------------------------
+# a stack normed behind the residual sum; an embedding with a hashed pair table
+# ----------------------------------------------------------------------------
+
+
+def embed_pair_hash(
+    table: torch.Tensor, pairs: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, token_request: torch.Tensor,
+    cu_seqlens_q: torch.Tensor, state_slots: torch.Tensor, last_token: torch.Tensor, *, mul_prev: int, mul_cur: int,
+    want_cast: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """`float32(table[ids]) + pairs[row]`, `row = (prev * mul_prev + id * mul_cur) mod buckets` where
+    `prev` is the token before in the same sequence, and `buckets` (the last row of `pairs`
+    [buckets + 1, H]) for a sequence's first token.  The token before a request's first token of
+    this step is read from `last_token` [slots + 1, >= 1] (int32, one row a state slot, the last row
+    nobody's) at the request's slot, and the request's last token of the step is left there.
+    Returns the float32 stream [T, H] and, with `want_cast`, the same rows in the table's dtype."""
+    _need_cuda(table, pairs, ids, positions, token_request, cu_seqlens_q, state_slots, last_token)
+    for name, t in (("table", table), ("pairs", pairs), ("ids", ids), ("positions", positions), ("token_request", token_request),
+                    ("cu_seqlens_q", cu_seqlens_q), ("state_slots", state_slots)):
+        _need_contiguous(name, t)
+    for name, t in (("ids", ids), ("positions", positions), ("token_request", token_request), ("cu_seqlens_q", cu_seqlens_q),
+                    ("state_slots", state_slots), ("last_token", last_token)):
+        _need_int32(name, t)
+    vocab, hidden = table.shape
+    if pairs.dim() != 2 or pairs.shape[1] != hidden or pairs.shape[0] < 2 or pairs.dtype != table.dtype:
+        raise KernelShapeError(f"embed_pair_hash: the pair table must be {table.dtype} [buckets + 1, {hidden}], got {pairs.dtype} {tuple(pairs.shape)}")
+    tokens = ids.numel()
+    if positions.numel() != tokens or token_request.numel() != tokens:
+        raise KernelShapeError("embed_pair_hash: one position and one request per token id")
+    if state_slots.numel() + 1 != cu_seqlens_q.numel():
+        raise KernelShapeError("embed_pair_hash: one state slot per request")
+    if last_token.dim() < 1 or last_token.shape[0] < 2:
+        raise KernelShapeError("embed_pair_hash: the state rows are [slots + 1, ...]")
+    out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    cast = torch.empty((tokens, hidden), dtype=table.dtype, device=table.device) if want_cast else None
+    library.check(
+        library.load().mi_embed_pair_hash(
+            _dtype_code(table), _ptr(table), _ptr(pairs), _ptr(ids), _ptr(positions), _ptr(token_request), _ptr(cu_seqlens_q),
+            _ptr(state_slots), _ptr(last_token), last_token.stride(0), last_token.shape[0] - 1, _ptr(out), _ptr(cast), tokens,
+            hidden, vocab, pairs.shape[0] - 1, int(mul_prev), int(mul_cur), _stream(),
+        )
+    )
+    return out, cast
+
+
+def scale_add_norm(
+    residual: torch.Tensor, y: torch.Tensor | None, scale: torch.Tensor | None, factor: torch.Tensor, alpha: float,
+    eps: float, dtype: torch.dtype, rows: torch.Tensor | None = None, want_cast: bool = True,
+) -> torch.Tensor | None:
+    """The norm behind the sum: `x <- rms_norm(alpha * x + scale * y) * factor` row by row, in place
+    on the float32 stream `residual` [T, H] (`scale`, `factor` float32 [H]; without `scale` the sum
+    is `alpha * x + y`; without `y` the row is normed as it is).  With `want_cast` the new rows are
+    returned in `dtype` as well.  With `rows` (int32) only those rows are normed, the stream stays
+    as it was and the normed rows come back [len(rows), H]."""
+    _need_cuda(residual, y, scale, factor, rows)
+    for name, t in (("residual", residual), ("scale", scale), ("factor", factor), ("rows", rows)):
+        _need_contiguous(name, t)
+    _need_f32("residual", residual)
+    _need_f32("scale", scale)
+    _need_f32("factor", factor)
+    _need_int32("rows", rows)
+    tokens, hidden = residual.shape
+    if y is not None and (y.dim() != 2 or y.stride(1) != 1 or tuple(y.shape) != (tokens, hidden) or y.dtype != dtype):
+        raise KernelShapeError(f"scale_add_norm: y {tuple(y.shape)} {y.dtype} does not fit the stream {(tokens, hidden)} in {dtype}")
+    if factor.numel() != hidden or (scale is not None and scale.numel() != hidden):
+        raise KernelShapeError(f"scale_add_norm: one factor (and one scale) per column of {hidden}")
+    if rows is not None and y is not None:
+        raise KernelShapeError("scale_add_norm: rows are picked for the norm alone")
+    count = tokens if rows is None else rows.numel()
+    cast = torch.empty((count, hidden), dtype=dtype, device=residual.device) if (want_cast or rows is not None) else None
+    library.check(
+        library.load().mi_scale_add_norm(
+            F32 if dtype == torch.float32 else BF16, _ptr(residual), _ptr(y), 0 if y is None else y.stride(0), _ptr(scale),
+            _ptr(factor), _ptr(rows), _ptr(cast), count, hidden, float(alpha), float(eps), _stream(),
+        )
+    )
+    return cast
+
+
+def norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, width: int | None = None) -> torch.Tensor:
+    """`x[:, :width] * rsqrt(mean(x[:, :width]^2) + eps) * weight` row by row -> [T, width] in the dtype of
+    `x` (`weight` float32 [width]; rows of `x` may be wider and strided)."""
+    _need_cuda(x, weight)
+    _need_contiguous("weight", weight)
+    _need_f32("weight", weight)
+    width = x.shape[1] if width is None else int(width)
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < width or weight.numel() != width:
+        raise KernelShapeError(f"norm_rows: rows of at least {width} columns and as many weights, got {tuple(x.shape)} and {weight.numel()}")
+    out = torch.empty((x.shape[0], width), dtype=x.dtype, device=x.device)
+    library.check(
+        library.load().mi_norm_rows(_dtype_code(x), _ptr(x), x.stride(0), _ptr(weight), _ptr(out), out.stride(0), x.shape[0],
+                                    width, float(eps), _stream())
+    )
+    return out
+
+
+def qkv_norm_write(
+    qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor | None, slot_mapping: torch.Tensor | None,
+    k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, *, q_width: int, kv_heads: int, head_dim: int,
+    v_head_dim: int, eps: float, v_transposed: bool = False, other_values: torch.Tensor | None = None,
+    mix: torch.Tensor | None = None,
+) -> None:
+    """`qkv` [T, q_width + kv_heads*head_dim + kv_heads*v_head_dim]: q is normed in place over its
+    whole width (`q * rsqrt(mean(q^2) + eps) * q_weight`); k, normed the same way with `k_weight`,
+    goes to its key-page slot; v goes to its value-page slot, as it is or, with `other_values`
+    [T, kv_heads*v_head_dim] (another layer's values of the same tokens) and `mix` (one float32),
+    as `(1 - mix) * v + mix * other_values`.  `kv_heads=0`: q only."""
+    _need_cuda(qkv, q_weight, k_weight, slot_mapping, k_pages, v_pages, other_values, mix)
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight), ("slot_mapping", slot_mapping),
+                    ("k_pages", k_pages), ("v_pages", v_pages)):
+        _need_contiguous(name, t)
+    _need_int32("slot_mapping", slot_mapping)
+    _need_f32("q_weight", q_weight)
+    _need_f32("k_weight", k_weight)
+    _need_f32("mix", mix)
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < q_width + kv_heads * (head_dim + v_head_dim):
+        raise KernelShapeError(f"qkv_norm_write: rows hold q, k and v, got {tuple(qkv.shape)} strides {qkv.stride()}")
+    if q_weight.numel() != q_width or (kv_heads > 0 and (k_weight is None or k_weight.numel() != kv_heads * head_dim)):
+        raise KernelShapeError("qkv_norm_write: one norm weight per column of q and of k")
+    tokens = qkv.shape[0]
+    page_size = num_pages = 0
+    if kv_heads > 0:
+        if slot_mapping is None or k_pages is None or v_pages is None:
+            raise KernelShapeError("writing keys and values needs slot_mapping, k_pages and v_pages")
+        if k_pages.dtype != qkv.dtype or v_pages.dtype != qkv.dtype:
+            raise KernelShapeError(f"pages are {k_pages.dtype}, activations {qkv.dtype}")
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelShapeError(f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}")
+        _check_v_pages(k_pages, v_pages, v_transposed, v_head_dim)
+        if slot_mapping.numel() != tokens:
+            raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    if other_values is not None:
+        if mix is None or mix.numel() != 1:
+            raise KernelShapeError("qkv_norm_write: values to mix in come with one float32 weight")
+        if (other_values.dim() != 2 or other_values.stride(1) != 1 or other_values.dtype != qkv.dtype
+                or tuple(other_values.shape) != (tokens, kv_heads * v_head_dim)):
+            raise KernelShapeError(f"qkv_norm_write: the other values must be {qkv.dtype} [{tokens}, {kv_heads * v_head_dim}], got {tuple(other_values.shape)}")
+    library.check(
+        library.load().mi_qkv_norm_write(
+            _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(q_weight), _ptr(k_weight), _ptr(other_values),
+            0 if other_values is None else other_values.stride(0), _ptr(mix) if other_values is not None else None,
+            _ptr(slot_mapping) if kv_heads > 0 else None, _ptr(k_pages) if kv_heads > 0 else None,
+            _ptr(v_pages) if kv_heads > 0 else None, tokens, q_width, kv_heads, head_dim, v_head_dim, page_size, num_pages,
+            int(v_transposed), float(eps), _stream(),
+        )
+    )
+
+
+# ----------------------------------------------------------------------------
+# routed experts
+# ----------------------------------------------------------------------------
+
+ROUTER_MAX_OUTPUTS = 1024
+
+
+def route_top_k(
+    x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, gate_row: torch.Tensor | None, *, top: int,
+    route_scale: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """Per row of `x` [T, W]: scores `softmax(router @ x)` over all router outputs (`router` float32
+    [outputs, W]), the `top` outputs with the largest `score + correction` (`correction` float32
+    [outputs] or None; the lower index wins a tie) -> their indices int32 [T, top] and weights
+    `score * route_scale` float32 [T, top] (not renormalized); with `gate_row` (float32 [W]) also
+    `logistic(gate_row . x)` float32 [T]."""
+    _need_cuda(x, router, correction, gate_row)
+    for name, t in (("router", router), ("correction", correction), ("gate_row", gate_row)):
+        _need_contiguous(name, t)
+        _need_f32(name, t)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelShapeError("route_top_k: rows with unit inner stride")
+    tokens, width = x.shape
+    if router.dim() != 2 or router.shape[1] != width:
+        raise KernelShapeError(f"route_top_k: the router is [outputs, {width}], got {tuple(router.shape)}")
+    outputs = router.shape[0]
+    if not 0 < top <= outputs or outputs > ROUTER_MAX_OUTPUTS:
+        raise KernelShapeError(f"route_top_k: {top} of {outputs} outputs (at most {ROUTER_MAX_OUTPUTS})")
+    if correction is not None and correction.numel() != outputs:
+        raise KernelShapeError(f"route_top_k: one correction per router output, got {correction.numel()} for {outputs}")
+    if gate_row is not None and gate_row.numel() != width:
+        raise KernelShapeError(f"route_top_k: the gate row has {gate_row.numel()} entries for {width} columns")
+    chosen = torch.empty((tokens, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=x.device)
+    gates = torch.empty((tokens,), dtype=torch.float32, device=x.device) if gate_row is not None else None
+    library.check(
+        library.load().mi_route_top_k(
+            _dtype_code(x), _ptr(x), x.stride(0), _ptr(router), _ptr(correction), _ptr(gate_row), _ptr(chosen), _ptr(weights),
+            _ptr(gates), tokens, width, outputs, int(top), float(route_scale), _stream(),
+        )
+    )
+    return chosen, weights, gates
+
+
+def _check_experts(x, gate_up, down, chosen, weights, shared, shared_gate):
+    _need_cuda(x, gate_up, down, chosen, weights, shared, shared_gate)
+    for name, t in (("gate_up", gate_up), ("down", down), ("chosen", chosen), ("weights", weights), ("shared_gate", shared_gate)):
+        _need_contiguous(name, t)
+    _need_int32("chosen", chosen)
+    _need_f32("weights", weights)
+    _need_f32("shared_gate", shared_gate)
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelShapeError("routed experts: rows with unit inner stride")
+    tokens, width = x.shape
+    if gate_up.dim() != 3 or down.dim() != 3 or gate_up.shape[2] != width or gate_up.shape[1] % 2 or gate_up.dtype != x.dtype or down.dtype != x.dtype:
+        raise KernelShapeError(f"routed experts: gate|up is {x.dtype} [experts, 2*ff, {width}], got {gate_up.dtype} {tuple(gate_up.shape)}")
+    experts, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    if tuple(down.shape) != (experts, width, ff):
+        raise KernelShapeError(f"routed experts: down is [{experts}, {width}, {ff}], got {tuple(down.shape)}")
+    if chosen.dim() != 2 or chosen.shape[0] != tokens or tuple(weights.shape) != tuple(chosen.shape):
+        raise KernelShapeError("routed experts: chosen and weights are [T, top]")
+    if shared is not None and (shared.dim() != 2 or shared.stride(1) != 1 or tuple(shared.shape) != (tokens, width) or shared.dtype != x.dtype
+                               or shared_gate is None or shared_gate.numel() != tokens):
+        raise KernelShapeError("routed experts: a shared expert's rows are [T, W] and come with one gate a row")
+    return tokens, width, experts, ff, chosen.shape[1]
+
+
+def experts_few_rows(
+    x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+    shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """`y[t] = sum_k weights[t, k] * expert_{chosen[t, k]}(x[t]) (+ shared_gate[t] * shared[t])` with
+    every (row, chosen expert) pair worked on its own, the expert's weights read by index: two
+    launches whatever the rows hold, and nothing the host has to know.  An index past the real
+    experts is an identity expert (its output is `x[t]`).  `gate_up` [experts, 2*ff, W] (gate rows,
+    then up rows), `down` [experts, W, ff]; an expert is `down(silu(gate(x)) * up(x))`."""
+    tokens, width, experts, ff, top = _check_experts(x, gate_up, down, chosen, weights, shared, shared_gate)
+    act = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
+    out = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
+    lib = library.load()
+    library.check(lib.mi_expert_gate_up(_dtype_code(x), _ptr(x), x.stride(0), _ptr(gate_up), _ptr(chosen), _ptr(act), tokens,
+                                        width, ff, experts, top, _stream()))
+    library.check(lib.mi_expert_down_combine(
+        _dtype_code(x), _ptr(act), _ptr(down), _ptr(chosen), _ptr(weights), _ptr(x), x.stride(0), _ptr(shared),
+        0 if shared is None else shared.stride(0), _ptr(shared_gate), _ptr(out), tokens, width, ff, experts, top, _stream()))
+    return out
+
+
+def experts_grouped(
+    x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+    shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """The same sum for many rows: the (row, expert) pairs are sorted by expert, every expert that
+    was chosen runs its two products once over all its rows (the engine's own products, so each
+    expert's weights are read once), and one kernel adds a row's results in the order of its
+    choices.  The host reads how many rows each expert got, so this form is not for a step that
+    is being recorded."""
+    tokens, width, experts, ff, top = _check_experts(x, gate_up, down, chosen, weights, shared, shared_gate)
+    flat = chosen.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=experts)[:experts].tolist()
+    sorted_rows = x.index_select(0, torch.div(order, top, rounding_mode="floor"))
+    where = torch.empty_like(order, dtype=torch.int32)
+    where[order] = torch.arange(order.numel(), dtype=torch.int32, device=x.device)
+    made, at = [], 0
+    for e, count in enumerate(counts):
+        if count:
+            made.append(linear(linear_swiglu(sorted_rows[at:at + count], gate_up[e]), down[e]))
+            at += count
+    rows = torch.cat(made, dim=0) if made else torch.empty((1, width), dtype=x.dtype, device=x.device)
+    out = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
+    library.check(library.load().mi_expert_combine(
+        _dtype_code(x), _ptr(rows), _ptr(where), _ptr(chosen), _ptr(weights), _ptr(x), x.stride(0), _ptr(shared),
+        0 if shared is None else shared.stride(0), _ptr(shared_gate), _ptr(out), tokens, width, experts, top, _stream()))
+    return out

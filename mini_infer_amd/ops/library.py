@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 31
+ABI_VERSION = 32
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -58,7 +58,7 @@ _SIGNATURES: dict[str, list] = {
     ],
     "mi_attn_mfma": [
         _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
-        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
+        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P, _P,
     ],
     "mi_gemm_skinny_addnorm_pieces": [c_int],
     "mi_gemm_skinny_addnorm_bf16": [
@@ -81,7 +81,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_gated_table_rows": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
     "mi_attn_general": [
         c_int, _P, c_int64, _P, _P, _P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, c_int,
-        c_int64, c_int, c_int, c_float, c_int, c_int, _P, c_int, c_float, c_int, _P,
+        c_int64, c_int, c_int, c_float, c_int, c_int, _P, c_int, c_float, c_int, c_float, _P, _P,
     ],
     "mi_stream_update_norm": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_float, _P],
     "mi_clamped_glu": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_float, _P],
@@ -93,11 +93,11 @@ _SIGNATURES: dict[str, list] = {
     "mi_gated_delta_rows": [c_int, c_int],
     "mi_latent_prepare": [
         c_int, _P, c_int64, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int,
-        c_float, _P,
+        c_float, _P, c_int64, _P,
     ],
     "mi_latent_expand": [
         c_int, _P, c_int64, c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
-        c_int, _P,
+        c_int, _P, c_int64, _P,
     ],
     "mi_embed_norm_streams": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
     "mi_streams_update_norm": [
@@ -114,6 +114,17 @@ _SIGNATURES: dict[str, list] = {
         c_int, c_int, _P,
     ],
     "mi_gated_mul": [c_int, c_int, _P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, _P],
+    "mi_embed_pair_hash": [c_int, _P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    "mi_scale_add_norm": [c_int, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_float, c_float, _P],
+    "mi_norm_rows": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, _P],
+    "mi_qkv_norm_write": [
+        c_int, _P, c_int64, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+        c_float, _P,
+    ],
+    "mi_route_top_k": [c_int, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P],
+    "mi_expert_gate_up": [c_int, _P, c_int64, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "mi_expert_down_combine": [c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, c_int, _P],
+    "mi_expert_combine": [c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
 }
 
 

@@ -317,6 +317,134 @@ class KeysAsValuesAttention(GQAttention):
         return self._project(self._attend(qk, ctx, cache))
 
 
+class WholeNormAttention(GQAttention):
+    """Grouped-query attention whose queries and keys are RMS-normed over their WHOLE projection
+    (all heads at once, one plain weight per column) before they are split into heads, with
+    values of their own and, each optional:
+
+    * `softcap`: a scaled score s becomes `softcap * tanh(s / softcap)` before anything else is done to it;
+    * `position`: any encoding; one that gives `score_slopes` takes `slope_h * distance` off the capped score;
+    * `learned_sink`: the softmax's denominator holds `exp(sink_h)` too, `sink_h` a learned number
+      per query head (tensor `sink_name`); it has no key and no value and is neither scaled nor capped;
+    * `value_mix` = {"key": k, "source": bool, "name": n}: layers that name the same key share values.
+      The source layer leaves its values of the step's tokens where the others find them; every
+      other layer caches `(1 - m) v + m v_source` of the same token, `m` its own learned number
+      (tensor `n`; the source's own is not read).
+
+    What is cached is the normed key and the (mixed) value, so decoding reads them as they are."""
+
+    can_defer_output = False
+    takes_scaled_rows = False
+
+    def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, position, dtype, device, *, norm_eps: float,
+                 v_head_dim=None, window=None, scale=None, names=("q", "k", "v", "o"), suffix="",
+                 norm_names=("q.norm", "k.norm"), softcap: float | None = None, learned_sink: bool = False,
+                 sink_name: str = "sink", value_mix: dict | None = None) -> None:
+        super().__init__(hidden_size, num_heads, num_kv_heads, head_dim, position, dtype, device, window=window,
+                         scale=scale, names=names, suffix=suffix, v_head_dim=v_head_dim)
+        if softcap is not None and not softcap > 0:
+            raise ValueError(f"a cap on the scores must be positive, got {softcap}")
+        if position is not None and position.rotary_layout() is not None:
+            raise NotImplementedError("attention normed over the whole projection with a rotation on top; not built")
+        self.norm_eps, self.norm_names = float(norm_eps), tuple(norm_names)
+        self.softcap = None if softcap is None else float(softcap)
+        self.learned_sink, self.sink_name = bool(learned_sink), sink_name
+        self.mix_key = None if value_mix is None else ("value_mix", str(value_mix["key"]))
+        self.mix_source = bool(value_mix["source"]) if value_mix is not None else False
+        self.mix_name = None if value_mix is None else str(value_mix.get("name", "vmix"))
+        self.q_norm: torch.Tensor | None = None
+        self.k_norm: torch.Tensor | None = None
+        self.sinks: torch.Tensor | None = None
+        self.mix: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        q_width, kv_width = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        specs = {
+            **super().param_specs(prefix),
+            prefix + self.norm_names[0]: ParamSpec((q_width,), init="norm_weight", dtype="float32"),
+            prefix + self.norm_names[1]: ParamSpec((kv_width,), init="norm_weight", dtype="float32"),
+        }
+        if self.learned_sink:
+            specs[prefix + self.sink_name] = ParamSpec((self.num_heads,), dtype="float32")
+        if self.mix_key is not None and not self.mix_source:
+            specs[prefix + self.mix_name] = ParamSpec((), dtype="float32")
+        return specs
+
+    def optional_names(self, prefix: str) -> set[str]:
+        return {prefix + self.mix_name} if self.mix_key is not None and self.mix_source else set()
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        super().load_params(prefix, get)
+        self.q_norm = get(prefix + self.norm_names[0]).float().contiguous()
+        self.k_norm = get(prefix + self.norm_names[1]).float().contiguous()
+        if self.learned_sink:
+            self.sinks = get(prefix + self.sink_name).float().contiguous()
+        if self.mix_key is not None and not self.mix_source:
+            self.mix = get(prefix + self.mix_name).float().reshape(1).contiguous()
+
+    def wants_scaled_rows(self, rows: int) -> bool:
+        return False
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        # (scores that are capped or biased by the distance run the plain kernel, which reads
+        # value pages that are not transposed)
+        v_head_dim = None if self.v_head_dim == self.head_dim else self.v_head_dim
+        return CacheNeeds(pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_head_dim=v_head_dim))
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None
+        assert self.qkv.weight is not None and self.q_norm is not None, "attention used before its weights were loaded"
+        if isinstance(x, ops.ScaledRows):
+            x = x.finish()
+        q_width, k_width = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        v_width = self.num_kv_heads * self.v_head_dim
+        other = None
+        if writes_cache:
+            qkv = self.qkv.forward(x)
+            kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
+            if self.mix_key is not None:
+                values = qkv[:, q_width + k_width: q_width + k_width + v_width]
+                if self.mix_source:
+                    ctx.shared[self.mix_key] = values  # (a view: the projection's rows stay as they are)
+                else:
+                    other = ctx.shared.get(self.mix_key)
+                    if other is None:
+                        raise RuntimeError("a layer that mixes values in ran before the layer whose values it mixes in")
+        else:
+            if self.mix_key is not None:
+                raise NotImplementedError("a layer that shares values and reads another call's cache; not built")
+            qkv = ops.linear(x, self.qkv.weight[:q_width])
+            kv_heads, slots = 0, None
+        ops.qkv_norm_write(
+            qkv, self.q_norm, self.k_norm if writes_cache else None, slots, cache.k_pages, cache.v_pages,
+            q_width=q_width, kv_heads=kv_heads, head_dim=self.head_dim, v_head_dim=self.v_head_dim, eps=self.norm_eps,
+            v_transposed=cache.v_transposed, other_values=other, mix=self.mix,
+        )
+        attended = ops.paged_attention(
+            qkv, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
+            ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
+            kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+            max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, slopes=self.slopes,
+            v_head_dim=self.v_head_dim, sinks=self.sinks, softcap=self.softcap,
+        )
+        return self.out.forward(attended)
+
+
+@register_mixer("whole_norm_attention")
+def build_whole_norm_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> WholeNormAttention:
+    position = None
+    pos_desc = desc.get("position")
+    if pos_desc is not None:
+        position = POSITION_ENCODINGS.lookup(pos_desc["kind"])(pos_desc, dtype, device, shared)
+    extra = {k: desc[k] for k in ("suffix", "v_head_dim", "softcap", "learned_sink", "sink_name", "value_mix", "norm_names") if k in desc}
+    if "names" in desc:
+        extra["names"] = tuple(desc["names"])
+    return WholeNormAttention(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["num_kv_heads"]), int(desc["head_dim"]), position, dtype,
+        device, norm_eps=float(desc["norm_eps"]), window=desc.get("window"), scale=desc.get("scale"), **extra,
+    )
+
+
 @register_mixer("keys_as_values_attention")
 def build_keys_as_values_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> KeysAsValuesAttention:
     extra = {k: desc[k] for k in ("names", "suffix", "norm_names") if k in desc}

@@ -206,6 +206,20 @@ class Norm(Part):
     ) -> torch.Tensor:
         raise NotImplementedError
 
+    def norm_sum(
+        self,
+        y: torch.Tensor,
+        residual: torch.Tensor,
+        scale: torch.Tensor | None = None,
+        alpha: float = 1.0,
+        want_cast: bool = False,
+    ) -> torch.Tensor | None:
+        """A third place a norm can stand: BEHIND the residual sum.  `residual <- norm(alpha *
+        residual + scale * y)` in place (float32; `scale` float32 [hidden] or None); with
+        `want_cast` the new rows are returned in the compute dtype too.  Only norms that a block
+        uses this way implement it."""
+        raise NotImplementedError(f"{type(self).__name__} cannot stand behind the residual sum")
+
     def add_output(
         self,
         y: torch.Tensor,
@@ -285,6 +299,10 @@ class Mixer(Part):
         (a mixer may choose its page layout by it)."""
         return CacheNeeds()
 
+    def optional_names(self, prefix: str) -> set[str]:
+        """Names a checkpoint may hold for this mixer without the mixer reading them."""
+        return set()
+
     def forward(
         self, x: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True
     ) -> torch.Tensor:
@@ -313,9 +331,17 @@ class FeedForward(Part):
 
 class Embedding(Part):
     """Starts the float32 residual stream of a step: `forward(ctx)` -> [T, hidden] float32
-    from `ctx.token_ids` (and, if it wishes, `ctx.positions`)."""
+    from `ctx.token_ids` (and, if it wishes, `ctx.positions`).
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    An embedding that has to remember something of a request from step to step (the token
+    before the step's first one, say) asks for state like a mixer does: `cache_needs` then
+    returns `CacheNeeds(state=...)` (no pages), the model lists it behind its layer calls' needs,
+    and `forward(ctx, cache)` is called with the `LayerCache` that holds its state rows."""
+
+    def cache_needs(self, page_size: int) -> "CacheNeeds | None":
+        return None
+
+    def forward(self, ctx: StepContext, cache: "LayerCache | None" = None) -> torch.Tensor:
         raise NotImplementedError
 
 

@@ -390,3 +390,95 @@ def build_hyper_connection_block(desc: dict, dtype: torch.dtype, device, shared:
         FEED_FORWARDS.lookup(ffn["kind"])(ffn, dtype, device, shared) if ffn is not None else None,
         int(desc.get("copies", 1)), bool(desc.get("learned", True)), dict(desc["names"]), dtype, device,
     )
+
+
+class PostNormBlock(Block):
+    """Sublayers that read the stream itself, which is normed BEHIND every sum:
+
+        x <- norm1(alpha * x + scale1 * mixer(x))
+        x <- norm2(alpha * x + scale2 * feed_forward(x))        (a layer may have none)
+
+    `scale1`, `scale2` are per-column layer scales (float32; a layer may have none), `alpha` one
+    number of the model.  Every sum is made here, by the norm's kernel (`Norm.norm_sum`), which also
+    leaves the stream's copy in the compute dtype for the next sublayer's products, so the block
+    hands nothing pending to what follows."""
+
+    takes_pending_products = False
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, feed_forward: FeedForward | None,
+                 hidden_size: int, alpha: float, layer_scale: bool, names: dict[str, str], dtype: torch.dtype, device) -> None:
+        super().__init__(dtype, device)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward = mixer_norm, mixer, ffn_norm, feed_forward
+        self.hidden_size, self.alpha, self.layer_scale, self.names = hidden_size, float(alpha), bool(layer_scale), names
+        self.mixer_scale: torch.Tensor | None = None
+        self.ffn_scale: torch.Tensor | None = None
+
+    def _children(self):
+        parts = [(self.names["mixer_norm"], self.mixer_norm), (self.names["mixer"], self.mixer)]
+        if self.feed_forward is not None:
+            parts += [(self.names["ffn_norm"], self.ffn_norm), (self.names["feed_forward"], self.feed_forward)]
+        return parts
+
+    @property
+    def graph_safe(self) -> bool:  # type: ignore[override]
+        return all(part.graph_safe for _, part in self._children())
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        specs: dict[str, ParamSpec] = {}
+        for sub, part in self._children():
+            specs.update(part.param_specs(prefix + sub))
+        if self.layer_scale:
+            specs[prefix + self.names["mixer_scale"]] = ParamSpec((self.hidden_size,), init="norm_weight", dtype="float32")
+            if self.feed_forward is not None:
+                specs[prefix + self.names["ffn_scale"]] = ParamSpec((self.hidden_size,), init="norm_weight", dtype="float32")
+        return specs
+
+    def optional_names(self, prefix: str) -> set[str]:
+        """A layer without a feed-forward has no use for the second norm and scale; a checkpoint
+        that stores them all the same is read without them."""
+        names = set(self.mixer.optional_names(prefix + self.names["mixer"])) if hasattr(self.mixer, "optional_names") else set()
+        if self.feed_forward is None:
+            names |= {prefix + self.names["ffn_norm"], prefix + self.names["ffn_scale"]}
+        return names
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        for sub, part in self._children():
+            part.load_params(prefix + sub, get)
+        if self.layer_scale:
+            self.mixer_scale = get(prefix + self.names["mixer_scale"]).float().contiguous()
+            if self.feed_forward is not None:
+                self.ffn_scale = get(prefix + self.names["ffn_scale"]).float().contiguous()
+
+    def forward(self, delta, residual: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        from mini_infer_amd.parts.embedding import STREAM_CAST, stream_for_products
+
+        if delta is not None:  # a block of another arrangement left its output to be added
+            residual.add_(delta.finish() if hasattr(delta, "finish") else delta)
+        narrow = self.dtype != torch.float32
+
+        def normed(cast):
+            if cast is not None:
+                ctx.shared[STREAM_CAST] = (residual, cast)
+
+        mixed = self.mixer.forward(stream_for_products(residual, ctx, self.dtype), ctx, cache, writes_cache)
+        normed(self.mixer_norm.norm_sum(mixed, residual, self.mixer_scale, self.alpha, narrow))
+        if self.feed_forward is not None:
+            fed = self.feed_forward.forward(stream_for_products(residual, ctx, self.dtype), ctx)
+            normed(self.ffn_norm.norm_sum(fed, residual, self.ffn_scale, self.alpha, narrow))
+        return None
+
+
+@register_block("post_norm")
+def build_post_norm_block(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> PostNormBlock:
+    """`desc`: `norm` (for both sublayers), `mixer`, optional `feed_forward`, `hidden_size`, `alpha`,
+    `layer_scale` (whether the layer has per-column scales) and `names` (each part's name inside the layer)."""
+    shared = {} if shared is None else shared
+    ffn = desc.get("feed_forward")
+    return PostNormBlock(
+        NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype, device, shared),
+        MIXERS.lookup(desc["mixer"]["kind"])(desc["mixer"], dtype, device, shared),
+        NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype, device, shared) if ffn is not None else None,
+        FEED_FORWARDS.lookup(ffn["kind"])(ffn, dtype, device, shared) if ffn is not None else None,
+        int(desc["hidden_size"]), float(desc.get("alpha", 1.0)), bool(desc.get("layer_scale", False)), dict(desc["names"]),
+        dtype, device,
+    )

@@ -15,7 +15,7 @@ from __future__ import annotations
 import torch
 
 from mini_infer_amd import ops
-from mini_infer_amd.parts.base import Embedding, Head, ParamSpec, StepContext, TensorGetter
+from mini_infer_amd.parts.base import CacheNeeds, Embedding, Head, LayerCache, ParamSpec, StateNeeds, StepContext, TensorGetter
 from mini_infer_amd.registry import register_embedding, register_head
 
 
@@ -35,7 +35,7 @@ class TokenEmbedding(Embedding):
     def load_params(self, prefix: str, get: TensorGetter) -> None:
         self.weight = get(prefix + self.name).contiguous()
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    def forward(self, ctx: StepContext, cache: LayerCache | None = None) -> torch.Tensor:
         assert self.weight is not None, "embedding used before its table was loaded"
         return ops.embed_gather(self.weight, ctx.token_ids)
 
@@ -47,7 +47,7 @@ class ScaledEmbedding(TokenEmbedding):
         super().__init__(vocab_size, hidden_size, name, dtype, device)
         self.scale = float(scale)
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    def forward(self, ctx: StepContext, cache: LayerCache | None = None) -> torch.Tensor:
         assert self.weight is not None, "embedding used before its table was loaded"
         return ops.embed_gather(self.weight, ctx.token_ids, self.scale)
 
@@ -83,7 +83,7 @@ class ScaledSinusoidEmbedding(TokenEmbedding):
         self.freq_host = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * pairs / hidden_size)
         self._freq: torch.Tensor | None = None
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    def forward(self, ctx: StepContext, cache: LayerCache | None = None) -> torch.Tensor:
         assert self.weight is not None, "embedding used before its table was loaded"
         if self._freq is None:
             self._freq = self.freq_host.to(self.device).contiguous()
@@ -190,7 +190,7 @@ class NormedStreamsEmbedding(TokenEmbedding):
         super().load_params(prefix, get)
         self.factor = (get(prefix + self.norm_name).float() + self.weight_offset).contiguous()
 
-    def forward(self, ctx: StepContext) -> torch.Tensor:
+    def forward(self, ctx: StepContext, cache: LayerCache | None = None) -> torch.Tensor:
         assert self.weight is not None and self.factor is not None, "embedding used before its tensors were loaded"
         return ops.embed_norm_streams(self.weight, ctx.token_ids, self.factor, self.copies, self.eps)
 
@@ -200,4 +200,53 @@ def build_normed_streams_embedding(desc: dict, dtype: torch.dtype, device, share
     return NormedStreamsEmbedding(
         int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), str(desc["norm_name"]), float(desc["eps"]),
         int(desc.get("copies", 1)), dtype, device, weight_offset=float(desc.get("weight_offset", 0.0)),
+    )
+
+
+class PairHashEmbedding(TokenEmbedding):
+    """`table[token]` plus a row of a second table chosen by the token AND the one before it:
+
+        row = (previous * mul_prev + token * mul_cur) mod buckets        (the table has buckets + 1 rows)
+
+    and the last row, number `buckets`, for a sequence's first token.  The token before a step's
+    first one belongs to the request's state: one int32 per request, asked of the cache manager
+    like a mixer's state (zeroed at admission, freed with the request, copied aside and put back
+    around a failing step), read and left behind by the kernel that gathers the rows."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, pair_name: str, buckets: int, mul_prev: int,
+                 mul_cur: int, dtype: torch.dtype, device) -> None:
+        super().__init__(vocab_size, hidden_size, name, dtype, device)
+        if buckets <= 0:
+            raise ValueError(f"a pair table needs a positive number of buckets, got {buckets}")
+        self.pair_name, self.buckets, self.mul_prev, self.mul_cur = pair_name, int(buckets), int(mul_prev), int(mul_cur)
+        self.pairs: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {**super().param_specs(prefix), prefix + self.pair_name: ParamSpec((self.buckets + 1, self.hidden_size))}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        super().load_params(prefix, get)
+        self.pairs = get(prefix + self.pair_name).contiguous()
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        return CacheNeeds(state=StateNeeds((1,), torch.int32))
+
+    def forward(self, ctx: StepContext, cache: LayerCache | None = None) -> torch.Tensor:
+        assert self.weight is not None and self.pairs is not None, "embedding used before its tables were loaded"
+        if cache is None or cache.state is None:
+            raise ValueError("a pair-hash embedding needs its state rows (the token before each request's next one)")
+        residual, cast = ops.embed_pair_hash(
+            self.weight, self.pairs, ctx.token_ids, ctx.positions, ctx.token_request, ctx.cu_seqlens_q, ctx.state_slots,
+            cache.state, mul_prev=self.mul_prev, mul_cur=self.mul_cur, want_cast=self.dtype != torch.float32,
+        )
+        if cast is not None:
+            ctx.shared[STREAM_CAST] = (residual, cast)
+        return residual
+
+
+@register_embedding("pair_hash_embedding")
+def build_pair_hash_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> PairHashEmbedding:
+    return PairHashEmbedding(
+        int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), str(desc["pair_name"]), int(desc["buckets"]),
+        int(desc["mul_prev"]), int(desc["mul_cur"]), dtype, device,
     )

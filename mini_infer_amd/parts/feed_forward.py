@@ -257,3 +257,115 @@ def build_clamped_gated_feed_forward(desc: dict, dtype: torch.dtype, device, sha
     if "names" in desc:
         extra["names"] = tuple(desc["names"])
     return ClampedGatedFeedForward(int(desc["hidden_size"]), int(desc["intermediate_size"]), float(desc["limit"]), dtype, device, **extra)
+
+
+class RoutedExperts(FeedForward):
+    """A mixture of experts: `experts` small gated feed-forwards (`W_down (silu(W_gate x) * W_up x)`, no
+    biases), of which every token goes through `top`.
+
+        z = R x (float32)        s = softmax(z) over ALL router outputs        choice = s + correction
+        y = sum over the `top` outputs e with the largest choice of  (s_e * route_scale) * expert_e(x)
+
+    The weights are the scores themselves (without the correction, not renormalized).  The last
+    `identity` router outputs stand for experts without tensors whose output is their input.  A
+    shared expert of the same form may run for every token beside them, gated by one number a
+    token, `logistic(w_sg . x)`.
+
+    Few rows (and every step that is recorded to be replayed) work each (token, expert) pair on its
+    own with the expert's weights read by index, two launches and nothing the host has to know;
+    many rows are sorted by expert and every chosen expert runs the engine's own products once over
+    all its rows.  Router, correction and the shared expert's gate row stay float32."""
+
+    graph_safe = True
+
+    # rows * top pairs, times the bytes of an expert, from which on sorting by expert pays for the
+    # launches of a loop over the experts (each pair reads its expert's weights once otherwise)
+    GROUPED_BYTES_PER_EXPERT = 64 << 20
+
+    def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, dtype: torch.dtype, device, *,
+                 identity: int = 0, route_scale: float = 1.0, correction: bool = True, shared_size: int | None = None,
+                 names: dict[str, str] | None = None) -> None:
+        super().__init__(dtype, device)
+        if experts <= 0 or identity < 0 or not 0 < top <= experts + identity:
+            raise ValueError(f"routed experts: {top} of {experts} experts + {identity} identity experts")
+        if experts + identity > ops.kernels.ROUTER_MAX_OUTPUTS:
+            raise ValueError(f"routed experts: the router takes at most {ops.kernels.ROUTER_MAX_OUTPUTS} outputs")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.experts, self.identity, self.top, self.route_scale = experts, identity, top, float(route_scale)
+        self.has_correction, self.shared_size = bool(correction), shared_size
+        self.names = {"router": "router", "correction": "correction", "expert": "e{}.", "gate": "gate", "up": "up",
+                      "down": "down", "shared": "shared.", "shared_gate": "shared.sg", **(names or {})}
+        self.shared = None if shared_size is None else SwiGLU(
+            hidden_size, shared_size, dtype, device,
+            names=tuple(self.names["shared"] + self.names[k] for k in ("gate", "up", "down")), suffix="")
+        if self.shared is not None:
+            self.shared.takes_scaled_rows = False
+        self.router: torch.Tensor | None = None  # float32 [experts + identity, hidden]
+        self.correction: torch.Tensor | None = None  # float32 [experts + identity]
+        self.shared_gate_row: torch.Tensor | None = None  # float32 [hidden]
+        self.gate_up: torch.Tensor | None = None  # [experts, 2 * ff, hidden]
+        self.down: torch.Tensor | None = None  # [experts, hidden, ff]
+        self.force_form: str | None = None  # "few" or "grouped": for tests and measurements
+
+    def _expert_name(self, prefix: str, e: int, which: str) -> str:
+        return prefix + self.names["expert"].format(e) + self.names[which]
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        outputs, ff, hidden = self.experts + self.identity, self.intermediate_size, self.hidden_size
+        specs = {prefix + self.names["router"]: ParamSpec((outputs, hidden), dtype="float32")}
+        if self.has_correction:
+            specs[prefix + self.names["correction"]] = ParamSpec((outputs,), dtype="float32")
+        for e in range(self.experts):
+            specs[self._expert_name(prefix, e, "gate")] = ParamSpec((ff, hidden))
+            specs[self._expert_name(prefix, e, "up")] = ParamSpec((ff, hidden))
+            specs[self._expert_name(prefix, e, "down")] = ParamSpec((hidden, ff))
+        if self.shared is not None:
+            specs.update(self.shared.param_specs(prefix))
+            specs[prefix + self.names["shared_gate"]] = ParamSpec((1, hidden), dtype="float32")
+        return specs
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.router = get(prefix + self.names["router"]).float().contiguous()
+        if self.has_correction:
+            self.correction = get(prefix + self.names["correction"]).float().contiguous()
+        ff, hidden = self.intermediate_size, self.hidden_size
+        first = get(self._expert_name(prefix, 0, "gate"))
+        self.gate_up = torch.empty((self.experts, 2 * ff, hidden), dtype=first.dtype, device=first.device)
+        self.down = torch.empty((self.experts, hidden, ff), dtype=first.dtype, device=first.device)
+        for e in range(self.experts):
+            self.gate_up[e, :ff] = get(self._expert_name(prefix, e, "gate"))
+            self.gate_up[e, ff:] = get(self._expert_name(prefix, e, "up"))
+            self.down[e] = get(self._expert_name(prefix, e, "down"))
+        if self.shared is not None:
+            self.shared.load_params(prefix, get)
+            self.shared_gate_row = get(prefix + self.names["shared_gate"]).float().reshape(-1).contiguous()
+
+    def _grouped(self, rows: int, ctx: StepContext) -> bool:
+        if self.force_form is not None:
+            return self.force_form == "grouped"
+        if ctx.host_cu_seqlens_q is None or torch.cuda.is_current_stream_capturing():
+            return False  # (the sorted form reads the experts' row counts on the host)
+        element = 2 if self.dtype == torch.bfloat16 else 4
+        expert_bytes = 3 * self.intermediate_size * self.hidden_size * element
+        return rows * self.top * expert_bytes > self.experts * self.GROUPED_BYTES_PER_EXPERT
+
+    def forward(self, x, ctx: StepContext) -> torch.Tensor:
+        assert self.router is not None and self.gate_up is not None and self.down is not None, \
+            "feed-forward used before its weights were loaded"
+        if hasattr(x, "finish"):
+            x = x.finish()
+        chosen, weights, gates = ops.route_top_k(x, self.router, self.correction, self.shared_gate_row, top=self.top,
+                                                 route_scale=self.route_scale)
+        shared = None
+        if self.shared is not None:
+            shared = self.shared.forward(x, ctx)
+            shared = shared.finish() if hasattr(shared, "finish") else shared
+        run = ops.experts_grouped if self._grouped(x.shape[0], ctx) else ops.experts_few_rows
+        return run(x, self.gate_up, self.down, chosen, weights, shared, gates)
+
+
+@register_feed_forward("routed_experts")
+def build_routed_experts(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> RoutedExperts:
+    extra = {k: desc[k] for k in ("identity", "route_scale", "correction", "shared_size", "names") if k in desc}
+    return RoutedExperts(int(desc["hidden_size"]), int(desc["intermediate_size"]), int(desc["experts"]), int(desc["top"]),
+                         dtype, device, **extra)

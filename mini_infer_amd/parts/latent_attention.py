@@ -40,7 +40,8 @@ from mini_infer_amd.parts.base import (
 from mini_infer_amd.parts.linear import Linear
 from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
 
-DEFAULT_NAMES = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "out": "o"}
+DEFAULT_NAMES = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "out": "o",
+                 "q_down": "dq", "q_down_norm": "dq.norm", "q_up": "uq", "sink": "sink"}
 
 
 class LatentAttention(Mixer):
@@ -48,8 +49,18 @@ class LatentAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, kv_rank: int,
                  position: PositionEncoding, scale: float, norm_eps: float, dtype: torch.dtype, device, *,
-                 names: dict[str, str] | None = None, suffix: str = "") -> None:
+                 names: dict[str, str] | None = None, suffix: str = "", q_rank: int | None = None, window: int | None = None,
+                 learned_sink: bool = False) -> None:
+        """`q_rank`: the queries go through a latent of their own, `q = W_uq rms_norm(W_dq h)` (tensors
+        `q_down`, `q_down_norm`, `q_up` of `names`) instead of one product `W_q h`.  `window`: position i
+        sees only the last `window` positions, itself included.  `learned_sink`: the softmax's
+        denominator holds `exp(sink_h)` too, `sink_h` a learned number per head (tensor `sink`)."""
         super().__init__(dtype, device)
+        if q_rank is not None and q_rank <= 0:
+            raise ValueError(f"latent attention: q_rank must be positive, got {q_rank}")
+        if window is not None and window <= 0:
+            raise ValueError(f"latent attention: the window must be positive, got {window}")
+        self.q_rank, self.window, self.learned_sink = q_rank, window, bool(learned_sink)
         for what, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim),
                             ("v_head_dim", v_head_dim), ("kv_rank", kv_rank)):
             if value <= 0:
@@ -70,9 +81,17 @@ class LatentAttention(Mixer):
         self.names = {**DEFAULT_NAMES, **(names or {})}
         n = self.names
         self.q_head_width = head_dim + rot_dim
-        # one product yields [q of every head | x_c | x_r]
-        self.q_down = Linear(hidden_size, [num_heads * self.q_head_width, kv_rank + rot_dim], [n["q"], n["down"]], dtype,
-                             device, suffix=suffix)
+        if q_rank is None:
+            # one product yields [q of every head | x_c | x_r]
+            self.q_down = Linear(hidden_size, [num_heads * self.q_head_width, kv_rank + rot_dim], [n["q"], n["down"]], dtype,
+                                 device, suffix=suffix)
+            self.q_up = None
+        else:
+            # one product yields [the queries' latent | x_c | x_r]; the queries are a second product
+            self.q_down = Linear(hidden_size, [q_rank, kv_rank + rot_dim], [n["q_down"], n["down"]], dtype, device, suffix=suffix)
+            self.q_up = Linear(q_rank, num_heads * self.q_head_width, n["q_up"], dtype, device, suffix=suffix)
+        self.q_latent_norm: torch.Tensor | None = None
+        self.sinks: torch.Tensor | None = None
         self.up_k = Linear(kv_rank, num_heads * head_dim, n["up_k"], dtype, device, suffix=suffix)
         self.up_v = Linear(kv_rank, num_heads * v_head_dim, n["up_v"], dtype, device, suffix=suffix)
         self.out = Linear(num_heads * v_head_dim, hidden_size, n["out"], dtype, device, suffix=suffix)
@@ -82,11 +101,17 @@ class LatentAttention(Mixer):
         self._out_padded: torch.Tensor | None = None  # W_o with zero columns where expanded value heads are padded
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
-        return {
+        specs = {
             **self.q_down.param_specs(prefix), **self.up_k.param_specs(prefix), **self.up_v.param_specs(prefix),
             **self.out.param_specs(prefix),
             prefix + self.names["down_norm"]: ParamSpec((self.kv_rank,), init="norm_weight", dtype="float32"),
         }
+        if self.q_up is not None:
+            specs.update(self.q_up.param_specs(prefix))
+            specs[prefix + self.names["q_down_norm"]] = ParamSpec((self.q_rank,), init="norm_weight", dtype="float32")
+        if self.learned_sink:
+            specs[prefix + self.names["sink"]] = ParamSpec((self.num_heads,), dtype="float32")
+        return specs
 
     def load_params(self, prefix: str, get: TensorGetter) -> None:
         self.q_down.load_params(prefix, get)
@@ -94,6 +119,11 @@ class LatentAttention(Mixer):
         self.up_v.load_params(prefix, get)
         self.out.load_params(prefix, get)
         self.latent_norm = get(prefix + self.names["down_norm"]).float().contiguous()
+        if self.q_up is not None:
+            self.q_up.load_params(prefix, get)
+            self.q_latent_norm = get(prefix + self.names["q_down_norm"]).float().contiguous()
+        if self.learned_sink:
+            self.sinks = get(prefix + self.names["sink"]).float().contiguous()
         assert self.up_k.weight is not None and self.up_v.weight is not None
         self.fold_k = self.up_k.weight.view(self.num_heads, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
         self.map_v = self.up_v.weight.view(self.num_heads, self.v_head_dim, self.kv_rank)
@@ -101,7 +131,7 @@ class LatentAttention(Mixer):
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
         # one key head, rows [c | r]; the values are the rows' front part: no value pages
-        return CacheNeeds(pages=PagedKVNeeds(1, self.kv_rank + self.rot_dim, None, v_head_dim=0))
+        return CacheNeeds(pages=PagedKVNeeds(1, self.kv_rank + self.rot_dim, self.window, v_head_dim=0))
 
     EXPAND_MIN_TOKENS = 64  # steps of fewer tokens take the folded form whatever they hold
 
@@ -140,18 +170,19 @@ class LatentAttention(Mixer):
             ctx.shared[key] = (both[: slots.size], both[slots.size:].view(table.shape), int(first[-1]))
         return ctx.shared[key]
 
-    def _forward_expanded(self, proj: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool) -> torch.Tensor:
+    def _forward_expanded(self, proj: torch.Tensor, down, c_col: int, ctx: StepContext, cache: LayerCache,
+                          writes_cache: bool) -> torch.Tensor:
         heads, rank, rot, dim, vdim = self.num_heads, self.kv_rank, self.rot_dim, self.head_dim, self.v_head_dim
         width, tokens = dim + rot, proj.shape[0]
         rotary = self.position.rotary(ctx)
         latent = torch.empty((tokens, rank), dtype=proj.dtype, device=proj.device)
         ops.latent_prepare(
             proj, rotary.cos, rotary.sin, self.latent_norm, ctx.slot_mapping[cache.group] if writes_cache else None,
-            cache.k_pages, None, heads=heads, q_head_width=self.q_head_width, q_rot_at=dim, c_col=heads * self.q_head_width,
-            rank=rank, rot=rot, eps=self.norm_eps, latent_out=latent,
+            cache.k_pages, None, heads=heads, q_head_width=self.q_head_width, q_rot_at=dim, c_col=c_col,
+            rank=rank, rot=rot, eps=self.norm_eps, latent_out=latent, down=down,
         )
         qkv = ops.latent_expand(proj, self.up_k.forward(latent), self.up_v.forward(latent), rotary.cos, rotary.sin, heads=heads,
-                                dim=dim, rot=rot, vdim=vdim, r_col=heads * self.q_head_width + rank)
+                                dim=dim, rot=rot, vdim=vdim, r_col=c_col + rank, down=down)
         slots, table, pages = self._own_pages(ctx)
         # (zeroed: the kernel multiplies what lies past a request's last key by a weight of zero)
         k_own = torch.zeros((pages, heads, ctx.page_size, width), dtype=proj.dtype, device=proj.device)
@@ -161,7 +192,8 @@ class LatentAttention(Mixer):
                           rotary_dim=0, v_transposed=True)
         mixed = ops.paged_attention(
             qkv, k_own, v_own, table, ctx.token_request, ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=heads,
-            kv_heads=heads, head_dim=width, scale=self.scale, window=None, max_seq_len=ctx.max_q_len, v_transposed=True,
+            kv_heads=heads, head_dim=width, scale=self.scale, window=self.window, max_seq_len=ctx.max_q_len, v_transposed=True,
+            sinks=self.sinks,
         )
         if self._out_padded is None:  # W_o with zero columns under the padding of every value head
             assert self.out.weight is not None
@@ -178,15 +210,21 @@ class LatentAttention(Mixer):
             x = x.finish()
         heads, rank, rot, width = self.num_heads, self.kv_rank, self.rot_dim, self.kv_rank + self.rot_dim
         proj = self.q_down.forward(x)
+        down, c_col = None, heads * self.q_head_width
+        if self.q_up is not None:
+            # [the queries' latent | x_c | x_r]: the latent is normed, and the queries are a product of their own
+            assert self.q_latent_norm is not None
+            down, c_col = proj, self.q_rank
+            proj = self.q_up.forward(ops.norm_rows(proj, self.q_latent_norm, self.norm_eps, width=self.q_rank))
         if self._expands(ctx):
-            return self._forward_expanded(proj, ctx, cache, writes_cache)
+            return self._forward_expanded(proj, down, c_col, ctx, cache, writes_cache)
         tokens = proj.shape[0]
         rotary = self.position.rotary(ctx)
         queries = torch.empty((tokens, heads * width), dtype=proj.dtype, device=proj.device)
         ops.latent_prepare(
             proj, rotary.cos, rotary.sin, self.latent_norm, ctx.slot_mapping[cache.group] if writes_cache else None,
             cache.k_pages, queries, heads=heads, q_head_width=self.q_head_width, q_rot_at=self.head_dim,
-            c_col=heads * self.q_head_width, rank=rank, rot=rot, eps=self.norm_eps,
+            c_col=c_col, rank=rank, rot=rot, eps=self.norm_eps, down=down,
         )
         # the key map folded into the queries: q'_a = W_uk,a^T q_a,plain
         plain = proj[:, : heads * self.q_head_width].unflatten(1, (heads, self.q_head_width))[:, :, : self.head_dim]
@@ -194,7 +232,7 @@ class LatentAttention(Mixer):
         mixed = ops.paged_attention(
             queries, cache.k_pages, None, ctx.block_tables[cache.group], ctx.token_request, ctx.positions,
             ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=heads, kv_heads=1, head_dim=width, scale=self.scale,
-            window=None, max_seq_len=ctx.max_seq_len, v_head_dim=rank,
+            window=self.window, max_seq_len=ctx.max_seq_len, v_head_dim=rank, sinks=self.sinks,
         )
         # the value map after the attention: W_uv,a (sum_j p_j c_j)
         values = torch.empty((tokens, heads * self.v_head_dim), dtype=proj.dtype, device=proj.device)
@@ -214,5 +252,6 @@ def build_latent_attention(desc: dict, dtype: torch.dtype, device, shared: dict 
     return LatentAttention(
         int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["head_dim"]), int(desc["rot_dim"]),
         int(desc["v_head_dim"]), int(desc["kv_rank"]), position, float(desc["scale"]), float(desc["norm_eps"]), dtype, device,
-        names=desc.get("names"), suffix=str(desc.get("suffix", "")),
+        names=desc.get("names"), suffix=str(desc.get("suffix", "")), q_rank=desc.get("q_rank"), window=desc.get("window"),
+        learned_sink=bool(desc.get("learned_sink", False)),
     )

@@ -163,3 +163,45 @@ class StreamsRMSNorm(Norm):
 def build_streams_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> StreamsRMSNorm:
     return StreamsRMSNorm(int(desc["hidden_size"]), float(desc["eps"]), int(desc.get("copies", 1)), dtype, device,
                           name=str(desc.get("name", "weight")), weight_offset=float(desc.get("weight_offset", 0.0)))
+
+
+class PostRMSNorm(Norm):
+    """RMS norm that stands BEHIND the residual sum: `x <- (alpha x + scale y) / rms(alpha x + scale y) *
+    (offset + w)`, the stream itself being what the norm left (`norm_sum`).  `weight_offset=1.0`
+    is a weight stored around zero.  As a model's last norm (`forward`) it norms the wanted rows of
+    the stream as they are.  Sum, statistics and the weight stay float32; the same launch leaves the
+    new rows in the compute dtype for the products that read them next."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device, name: str = "weight",
+                 weight_offset: float = 0.0) -> None:
+        super().__init__(dtype, device)
+        self.hidden_size, self.eps, self.name, self.weight_offset = hidden_size, float(eps), name, float(weight_offset)
+        self.factor: torch.Tensor | None = None  # float32 [H]: offset + weight
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        init = "norm_weight" if self.weight_offset == 0.0 else "normal"
+        return {prefix + self.name: ParamSpec((self.hidden_size,), init=init, dtype="float32")}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.factor = (get(prefix + self.name).float() + self.weight_offset).contiguous()
+
+    def norm_sum(self, y, residual, scale=None, alpha=1.0, want_cast=False):
+        assert self.factor is not None, "norm used before its weight was loaded"
+        y = y.finish() if hasattr(y, "finish") else y
+        return ops.scale_add_norm(residual, y, scale, self.factor, alpha, self.eps, self.dtype, want_cast=want_cast)
+
+    def forward(self, delta, residual: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
+        assert self.factor is not None, "norm used before its weight was loaded"
+        if delta is not None:  # a block of another arrangement left its output to be added
+            residual.add_(delta.finish() if hasattr(delta, "finish") else delta)
+        if rows is None:
+            rows = torch.arange(residual.shape[0], dtype=torch.int32, device=residual.device)
+        return ops.scale_add_norm(residual, None, None, self.factor, 1.0, self.eps, self.dtype, rows=rows)
+
+
+@register_norm("post_rms_norm")
+def build_post_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> PostRMSNorm:
+    return PostRMSNorm(int(desc["hidden_size"]), float(desc["eps"]), dtype, device, name=str(desc.get("name", "weight")),
+                       weight_offset=float(desc.get("weight_offset", 0.0)))

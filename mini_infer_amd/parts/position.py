@@ -125,3 +125,24 @@ def build_rotary(desc: dict, dtype: torch.dtype, device, shared: dict | None = N
         llama3=desc.get("llama3"),
         exact_frequencies=bool(desc.get("exact_frequencies", False)),
     )
+
+
+class DistanceSlopes(PositionEncoding):
+    """No rotation: positions enter the scores as a penalty linear in the distance, `slope_h * (i - j)`
+    taken off the score of query head h at position i for the key at position j, with slopes in a
+    geometric row, `slope_h = 2^(-total * (h + 1) / heads)` for h = 0 .. heads - 1."""
+
+    graph_safe = True
+
+    def __init__(self, total_exponent: float, dtype: torch.dtype, device) -> None:
+        super().__init__(dtype, device)
+        self.total_exponent = float(total_exponent)
+
+    def score_slopes(self, num_heads: int) -> torch.Tensor:
+        heads = torch.arange(1, num_heads + 1, dtype=torch.float64)
+        return torch.pow(2.0, -self.total_exponent * heads / num_heads).to(torch.float32).to(self.device).contiguous()
+
+
+@register_position_encoding("distance_slopes")
+def build_distance_slopes(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> DistanceSlopes:
+    return DistanceSlopes(float(desc.get("total_exponent", 8.0)), dtype, device)
