@@ -126,6 +126,10 @@ class KunudraConfig:
                 _count("embedding.bigram.mul_prev", section.get("mul_prev")),
                 _count("embedding.bigram.mul_cur", section.get("mul_cur")),
             )
+        parsed = tuple(_parse_layer(f"layers[{i}]", entry) for i, entry in enumerate(layers))
+        shared_widths = {layer.kv_heads * layer.vdim for layer in parsed if layer.v_mix}
+        if len(shared_widths) > 1:
+            raise ConfigError(f"layers that mix values share rows of one width, got kv_heads * vdim of {sorted(shared_widths)}")
         return cls(
             architecture=str(raw.get("architecture") or (raw.get("architectures") or [NAME])[0]),
             vocab=_positive_int("vocab", raw.get("vocab")),
@@ -133,7 +137,7 @@ class KunudraConfig:
             norm_eps=eps,
             alpha=_number("postln_alpha", raw.get("postln_alpha", 1.0)),
             pair_table=pair_table,
-            layers=tuple(_parse_layer(f"layers[{i}]", entry) for i, entry in enumerate(layers)),
+            layers=parsed,
         )
 
 

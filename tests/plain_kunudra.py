@@ -138,6 +138,11 @@ def gated_feed_forward(h: np.ndarray, w: dict, store=keep) -> np.ndarray:
     return store(store(silu(store(h @ w["gate"].T)) * store(h @ w["up"].T)) @ w["down"].T)
 
 
+# a list here collects, for every token of every routed layer, how far the last chosen expert's choice
+# score lies above the best one left out (a test can then keep to inputs whose choices no rounding turns)
+CHOICE_MARGINS: list | None = None
+
+
 def routed_feed_forward(x: np.ndarray, w: dict, mlp: dict, store=keep) -> np.ndarray:
     """Each token's `top` experts by score plus correction, weighted by the score itself times a
     constant; the last router outputs stand for experts that return their input; a shared expert
@@ -145,12 +150,16 @@ def routed_feed_forward(x: np.ndarray, w: dict, mlp: dict, store=keep) -> np.nda
     router = mlp["router"]
     experts, identity, top = router["experts"], router.get("identity", 0), router["top"]
     out = np.zeros_like(x)
+    margins = CHOICE_MARGINS
     for t in range(x.shape[0]):
         z = w["router"].astype(np.float64) @ x[t]
         s = np.exp(z - z.max())
         s = s / s.sum()
         choice = s + (w["correction"] if "correction" in w else 0.0)
-        for e in np.argsort(-choice, kind="stable")[:top]:
+        ranked = np.argsort(-choice, kind="stable")
+        if margins is not None and top < len(ranked):
+            margins.append(float(choice[ranked[top - 1]] - choice[ranked[top]]))
+        for e in ranked[:top]:
             weight = s[e] * router.get("scale", 1.0)
             if e >= experts:
                 assert e < experts + identity
