@@ -475,6 +475,36 @@ def kemurax_config(sizes: dict, layers: int) -> dict:
             "layers": [gla if i % 4 == 0 else pair for i in range(layers)]}
 
 
+KUNUDRA_EXPERTS = 16
+KUNUDRA_TOP = 2
+
+
+def kunudra_config(sizes: dict, layers: int) -> dict:
+    """A Kunudra model with the widths of a Llama configuration: latent attention, two layers of
+    grouped-query attention with capped scores, distance bias and shared values, latent attention, and
+    so on, all with a window of 1,024 keys and a sink per head; the first layer with a dense
+    feed-forward of Llama's width, every other layer with 16 experts a quarter as wide, of which a token
+    takes 2 of 16 + 2 identity experts, beside a shared expert of the same width.  The attention is
+    Llama's (heads, key/value heads, head size); the latent is four head sizes wide with half a head size
+    of rotated part, the queries' latent twelve head sizes (the proportions of published latent-attention
+    models)."""
+    h, heads, kv, d = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"], sizes["head_dim"]
+    ff = sizes["intermediate_size"]
+    window = {"size": DESIGN_WINDOW}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4},
+           "router": {"experts": KUNUDRA_EXPERTS, "identity": 2, "top": KUNUDRA_TOP, "scale": 1.5}}
+    attention = {"type": "attention",
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": window, "softcap": 50.0,
+                           "v_mix": True}}
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "kv_rank": 4 * d, "q_rank": 12 * d, "mask": window,
+                        "scale": (d + d // 2) ** -0.5, "rot": {"base": 10000.0, "dims": d // 2}}}
+    return {"architecture": "Kunudra", "vocab": sizes["vocab_size"], "width": h, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 7}},
+            "layers": [dict((latent, attention, attention, latent)[i % 4], mlp=dense if i == 0 else moe) for i in range(layers)]}
+
+
 def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
     """What a step must move and compute, from the model's own list of tensors: bytes of every matrix
     a decode step streams (tables that are only gathered from are left out), multiply-adds of its
@@ -502,6 +532,28 @@ def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
         # (the latent's key and value maps are applied per head to queries and outputs: counted with the matrices)
         return {"matrix_values": matrix, "kv_values_per_request": kv_values, "state_bytes_per_request": state_bytes,
                 "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops}
+    if raw.get("architecture") == "Kunudra":
+        # windowed attention: keys and values of every key/value head inside the window; latent attention:
+        # one row [latent | rotated part] per token inside the window; experts: a decode step streams only
+        # the experts its tokens chose (counted per batch by the caller: `expert_values` is one expert of
+        # every routed layer, `experts`/`top` how many there are and how many a token takes); the embedding
+        # table is the head
+        seen = lambda m: min(context, m["mask"]["size"]) if m.get("mask") else context  # noqa: E731
+        mixers = [(l["type"], l["mixer"]) for l in raw["layers"]]
+        routed = [l["mlp"] for l in raw["layers"] if l["mlp"] is not None and l["mlp"]["kind"] == "moe"]
+        expert_values = sum(3 * m["expert"]["ff"] * raw["width"] for m in routed)
+        all_experts = sum(m["router"]["experts"] * 3 * m["expert"]["ff"] * raw["width"] for m in routed)
+        matrix += head - all_experts - int(specs["bigram"].shape[0]) * int(specs["bigram"].shape[1])
+        kv_values = sum(m["kv_heads"] * (m["dim"] + m["vdim"]) * seen(m) for t, m in mixers if t == "attention")
+        kv_values += sum((m["kv_rank"] + m["rot_dim"]) * seen(m) for t, m in mixers if t == "latent_attention")
+        pairs = lambda m: sum(min(i + 1, m["mask"]["size"] if m.get("mask") else tokens) for i in range(tokens))  # noqa: E731
+        attention_flops = sum(2.0 * pairs(m) * m["heads"] * (m["dim"] + m["vdim"]) for t, m in mixers if t == "attention")
+        attention_flops += sum(2.0 * pairs(m) * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"]) for t, m in mixers if t == "latent_attention")
+        real_share = [m["router"]["experts"] / (m["router"]["experts"] + m["router"].get("identity", 0)) for m in routed]
+        expert_flops = sum(2.0 * tokens * m["router"]["top"] * share * 3 * m["expert"]["ff"] * raw["width"] for m, share in zip(routed, real_share))
+        return {"matrix_values": matrix, "kv_values_per_request": kv_values, "expert_values": expert_values,
+                "experts": KUNUDRA_EXPERTS, "top": KUNUDRA_TOP,
+                "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops + expert_flops}
     if raw.get("architecture") == "Kemurax":
         # attention inside chunks: a token sees the keys of its own chunk only; the recurrences keep a
         # float32 matrix per head (read and written once a step), the state-space layer also the last
@@ -583,7 +635,10 @@ def measure_model(raw: dict, dtype: str, batches: list[int], steps: int, warmup:
         seconds = (time.perf_counter() - started) / steps
         for rid in ids:
             runner.free_request(rid)
-        moved = (costs["matrix_values"] + batch * costs["kv_values_per_request"]) * elem + batch * costs.get("state_bytes_per_request", 0)
+        # (routed experts: a step streams the experts its tokens chose, at most all of them)
+        chosen_experts = min(costs.get("experts", 0), batch * costs.get("top", 0)) * costs.get("expert_values", 0)
+        moved = (costs["matrix_values"] + chosen_experts + batch * costs["kv_values_per_request"]) * elem \
+            + batch * costs.get("state_bytes_per_request", 0)
         out["decode"][f"b{batch}"] = {"ms_per_step": round(seconds * 1e3, 4), "tok_s": round(batch / seconds, 1),
                                       "frac_of_hbm_peak": round(moved / seconds / 1e9 / PEAK_HBM_GBS, 4)}
     del runner
@@ -602,6 +657,8 @@ def measure_design(design: str, sizes_name: str, dtype: str, layers: int | None,
         sides = [(design, zekonex_config(sizes, layers)), ("nadosun", nadosun_config(sizes, layers)), ("llama", theirs)]
     elif design == "kemurax":  # beside the design whose recurrent layers also keep a matrix per head, and beside Llama
         sides = [(design, kemurax_config(sizes, layers)), ("zekonex", zekonex_config(sizes, layers)), ("llama", theirs)]
+    elif design == "kunudra":  # beside the design that also has latent attention and attention with a sink, and beside Llama
+        sides = [(design, kunudra_config(sizes, layers)), ("zekonex", zekonex_config(sizes, layers)), ("llama", theirs)]
     else:
         raise ValueError(f"no design {design!r} to compare")
     line = {"design": design, "sizes": f"{model_name} layer sizes", "layers": layers, "dtype": dtype, "window": DESIGN_WINDOW,
@@ -649,10 +706,10 @@ def main() -> int:
                         help="with --serving / --reference-workload: launch steps that have portions of prompts in them kernel "
                         "by kernel, however few their tokens (recorded steps of single tokens stay)")
     parser.add_argument(
-        "--design", default=None, choices=("nadosun", "zekonex", "kemurax"),
+        "--design", default=None, choices=("nadosun", "zekonex", "kemurax", "kunudra"),
         help="instead of the default run: prefill (one 2,048-token prompt) and decode (batch 1, --batch and 64; --steps "
         "steps, default 64 here) of that design beside Llama at the layer sizes of --sizes and equal depth "
-        "(--layers, default 12; zekonex also beside nadosun, kemurax beside zekonex); prints one JSON line and exits",
+        "(--layers, default 12; zekonex also beside nadosun, kemurax and kunudra beside zekonex); prints one JSON line and exits",
     )
     parser.add_argument("--design-alone", action="store_true", help="with --design: leave the Llama side out (for profiles)")
     parser.add_argument("--attention-batch", type=int, default=0)

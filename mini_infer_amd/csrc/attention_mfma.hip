@@ -71,7 +71,7 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     float* __restrict__ part_ml, int q_heads, int kv_heads, int page_size_arg, unsigned page_magic, float scale_log2,
     int window, int num_splits, int heads_per_block, int tokens_per_tile, int one_tile_per_request,
     int pair_group, int first_token, int has_sink, float sink_log2, int mask_chunk,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, const float* __restrict__ slopes, float softcap) {
   constexpr int KSTEPS = D / 32;  // MFMA k-steps over the head dim for S^T
   // PS != 0: the page size is this constant (divisions become shifts, value offsets
   // immediates); PS == 0: any multiple of 16, divided by multiplying with
@@ -246,6 +246,14 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
   // scale) above which the reference has to move.
   float neg_ref[RG], raw_limit[RG];
   const float inv_scale_log2 = 1.f / scale_log2;
+  // scores that are capped or biased by the distance before the softmax (see block_softmax)
+  const bool shaped_scores = softcap > 0.f || slopes != nullptr;
+  const float scale_plain = scale_log2 / LOG2E;
+  const float cap_out = softcap > 0.f ? softcap / scale_plain : 0.f;             // the cap in raw units
+  const float cap_in = softcap > 0.f ? 2.f * LOG2E * scale_plain / softcap : 0.f;  // exp(2x) as exp2
+  float slope_raw[RG];
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) slope_raw[rg] = slopes != nullptr ? slopes[head[rg]] / scale_plain : 0.f;
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
@@ -363,6 +371,26 @@ __global__ __launch_bounds__(64 * WAVES * KW, OCC) void attn_mfma_kernel(
     // elsewhere hidden scores become -inf where they lie, before anything reads them (one
     // branch for all row groups, and no second copy of the scores for the two ways to merge in)
     const bool interior = kb >= interior_first && kb <= interior_last;
+    if (shaped_scores) {
+      // capped scores and a bias linear in the distance, on the raw scores where they lie, in the raw
+      // scores' own units (the scale comes later, with the exponential):
+      //   s <- (cap / scale) * tanh(s * scale / cap) - (slope / scale) * (pos - key)
+      // tanh(x) = 1 - 2 / (1 + exp(2x)) on the hardware's exponential and reciprocal (exact at both ends)
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = s_acc[rg][hlf][r];
+            if (softcap > 0.f) {
+              const float e = __builtin_amdgcn_exp2f(v * cap_in);
+              v = cap_out - 2.f * cap_out * __builtin_amdgcn_rcpf(1.f + e);
+            }
+            const int key = kb + 16 * hlf + 4 * quad + r;
+            s_acc[rg][hlf][r] = __builtin_fmaf(slope_raw[rg], (float)(key - pos[rg]), v);
+          }
+    }
     if (!interior) {
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg)
@@ -813,8 +841,9 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
                             int head_dim, int page_size, int num_pages, float scale, int window,
                             int num_splits, int shape, int one_tile_per_request,
                             int first_token, int combine, int has_sink, float sink_logit, int mask_chunk,
-                            const float* sinks, hipStream_t stream) {
+                            const float* sinks, const float* slopes, float softcap, hipStream_t stream) {
   MI_REQUIRE(sinks == nullptr || has_sink, "attn_mfma: per-head sink logits come with has_sink");
+  MI_REQUIRE(softcap >= 0.f, "attn_mfma: softcap=%g must be 0 (none) or positive", (double)softcap);
   MI_REQUIRE(mask_chunk >= 0, "attn_mfma: mask_chunk=%d must be 0 (none) or positive", mask_chunk);
   MI_REQUIRE(first_token >= 0, "attn_mfma: first_token=%d is negative", first_token);
   MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && num_tiles >= 0,
@@ -875,7 +904,7 @@ extern "C" int mi_attn_mfma(const void* q, int64_t q_row_stride, const void* k_p
       out_row_stride, part_acc, part_ml, q_heads, kv_heads, page_size, page_magic, scale_log2,    \
       window,                                                                                     \
       num_splits, hb, tq, one_tile_per_request, pair_group, first_token, has_sink, sink_logit * LOG2E, mask_chunk, \
-      sinks)
+      sinks, slopes, softcap)
 // (head sizes above 128 have no wide shape and were refused above: their cases name the 128 kernel,
 // so that nothing is compiled for them)
 #define MI_LAUNCH_P(DD, PP)                                                                       \

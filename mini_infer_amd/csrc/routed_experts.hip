@@ -43,33 +43,65 @@ __device__ __forceinline__ double exp_of(double z) { return exp(z); }
 
 #define MI_ROUTER_MAX_OUTPUTS 1024
 
-template <typename T>
-__global__ __launch_bounds__(256) void route_top_k_kernel(
+// R tokens a block: their rows wait in LDS while every wave walks router rows (16 bytes a lane, each
+// router row read once for all R tokens), then thread r ranks token r's outputs.
+template <typename T, int R>
+__global__ __launch_bounds__(1024) void route_top_k_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ router, const float* __restrict__ correction,
     const float* __restrict__ gate_row, int* __restrict__ chosen, float* __restrict__ weights,
-    float* __restrict__ shared_gate, int width, int outputs, int top, float route_scale) {
+    float* __restrict__ shared_gate, int num_tokens, int width, int outputs, int top, float route_scale) {
   using A = typename SumOf<T>::type;
-  __shared__ A z[MI_ROUTER_MAX_OUTPUTS + 1];
-  const int t = blockIdx.x;
-  const T* row = x + (int64_t)t * x_stride;
-  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE, waves = blockDim.x / MI_WAVE;
-  const int total = outputs + (gate_row != nullptr ? 1 : 0);
-  for (int e = wave; e < total; e += waves) {
-    const float* r = e < outputs ? router + (int64_t)e * width : gate_row;
-    A sum = 0;
-    for (int c = lane; c < width; c += MI_WAVE) sum += (A)r[c] * (A)to_f32(row[c]);
-    sum = lanes_total(sum);
-    if (lane == 0) z[e] = sum;
+  extern __shared__ __align__(16) unsigned char lds_bytes[];
+  A* z = reinterpret_cast<A*>(lds_bytes);                         // [R][outputs + 1]
+  T* rows = reinterpret_cast<T*>(z + (size_t)R * (outputs + 1));  // [R][width]
+  const int t0 = blockIdx.x * R;
+  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
+    const int r = i / width, c = i % width;
+    rows[i] = (t0 + r < num_tokens) ? x[(int64_t)(t0 + r) * x_stride + c] : from_f32<T>(0.f);
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  if (gate_row != nullptr) shared_gate[t] = (float)((A)1 / ((A)1 + exp_of(-z[outputs])));
-  A most = z[0];
-  for (int e = 1; e < outputs; ++e) most = z[e] > most ? z[e] : most;
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE, waves = blockDim.x / MI_WAVE;
+  const int total = outputs + (gate_row != nullptr ? 1 : 0);
+  const bool vec = width % 4 == 0 && ((uintptr_t)router % 16) == 0 && (gate_row == nullptr || ((uintptr_t)gate_row % 16) == 0);
+  for (int e = wave; e < total; e += waves) {
+    const float* w = e < outputs ? router + (int64_t)e * width : gate_row;
+    A sum[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) sum[r] = 0;
+    if (vec) {
+#pragma unroll 4
+      for (int c = lane * 4; c < width; c += MI_WAVE * 4) {
+        const float4 w4 = *reinterpret_cast<const float4*>(w + c);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const T* xr = rows + (size_t)r * width + c;
+          sum[r] += (A)w4.x * (A)to_f32(xr[0]) + (A)w4.y * (A)to_f32(xr[1]) + (A)w4.z * (A)to_f32(xr[2]) + (A)w4.w * (A)to_f32(xr[3]);
+        }
+      }
+    } else {
+      for (int c = lane; c < width; c += MI_WAVE) {
+        const A wc = (A)w[c];
+#pragma unroll
+        for (int r = 0; r < R; ++r) sum[r] += wc * (A)to_f32(rows[(size_t)r * width + c]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const A all = lanes_total(sum[r]);
+      if (lane == 0) z[r * (outputs + 1) + e] = all;
+    }
+  }
+  __syncthreads();
+  const int r = threadIdx.x, t = t0 + r;
+  if (r >= R || t >= num_tokens) return;
+  A* mine = z + r * (outputs + 1);
+  if (gate_row != nullptr) shared_gate[t] = (float)((A)1 / ((A)1 + exp_of(-mine[outputs])));
+  A most = mine[0];
+  for (int e = 1; e < outputs; ++e) most = mine[e] > most ? mine[e] : most;
   A sum = 0;
   for (int e = 0; e < outputs; ++e) {
-    z[e] = exp_of(z[e] - most);
-    sum += z[e];
+    mine[e] = exp_of(mine[e] - most);
+    sum += mine[e];
   }
   const A inv = (A)1 / sum;
   // the choice is made on score + correction, the weight is the score alone
@@ -77,13 +109,13 @@ __global__ __launch_bounds__(256) void route_top_k_kernel(
     int best = -1;
     A best_choice = 0;
     for (int e = 0; e < outputs; ++e) {
-      if (z[e] < (A)0) continue;  // taken already
-      const A choice = z[e] * inv + (correction != nullptr ? (A)correction[e] : (A)0);
+      if (mine[e] < (A)0) continue;  // taken already
+      const A choice = mine[e] * inv + (correction != nullptr ? (A)correction[e] : (A)0);
       if (best < 0 || choice > best_choice) best = e, best_choice = choice;
     }
     chosen[(int64_t)t * top + k] = best;
-    weights[(int64_t)t * top + k] = (float)(z[best] * inv * (A)route_scale);
-    z[best] = (A)-1;
+    weights[(int64_t)t * top + k] = (float)(mine[best] * inv * (A)route_scale);
+    mine[best] = (A)-1;
   }
 }
 
@@ -215,12 +247,27 @@ extern "C" int mi_route_top_k(int dtype, const void* x, int64_t x_stride, const 
   MI_REQUIRE(gate_row == nullptr || shared_gate != nullptr, "route_top_k: a gate row needs a place for the gates");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "route_top_k: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
-  if (dtype == MI_F32)
-    route_top_k_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)x, x_stride, router, correction, gate_row, chosen,
-                                                              weights, shared_gate, width, outputs, top, route_scale);
-  else
-    route_top_k_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)x, x_stride, router, correction, gate_row,
-                                                               chosen, weights, shared_gate, width, outputs, top, route_scale);
+  // as many tokens a block as fit its staging (rows in the element type, sums beside them), at most 4
+  const size_t elem = dtype == MI_F32 ? 4 : 2, acc = dtype == MI_F32 ? 8 : 4;
+  auto lds_for = [&](int r) { return (size_t)r * (outputs + 1) * acc + (size_t)r * width * elem; };
+  const int per_block = lds_for(4) <= 64 * 1024 ? 4 : (lds_for(2) <= 64 * 1024 ? 2 : 1);
+  MI_REQUIRE(lds_for(per_block) <= 64 * 1024, "route_top_k: rows of %d do not fit the block's staging", width);
+  const int threads = num_tokens <= 64 ? 1024 : 256;
+  const int blocks = ceil_div(num_tokens, per_block);
+#define MI_ROUTE(T, R)                                                                                               \
+  route_top_k_kernel<T, R><<<blocks, threads, lds_for(R), stream>>>((const T*)x, x_stride, router, correction, gate_row, \
+                                                                    chosen, weights, shared_gate, num_tokens, width,    \
+                                                                    outputs, top, route_scale)
+  if (dtype == MI_F32) {
+    if (per_block == 4) MI_ROUTE(float, 4);
+    else if (per_block == 2) MI_ROUTE(float, 2);
+    else MI_ROUTE(float, 1);
+  } else {
+    if (per_block == 4) MI_ROUTE(bf16_t, 4);
+    else if (per_block == 2) MI_ROUTE(bf16_t, 2);
+    else MI_ROUTE(bf16_t, 1);
+  }
+#undef MI_ROUTE
   MI_CHECK_LAUNCH("route_top_k");
   return MI_OK;
 }

@@ -925,15 +925,14 @@ def paged_attention(
 
     `sinks` (float32 [q_heads], optional): a sink logit per query head instead of one for all
     (both kernels).  `softcap`: every scaled score becomes `softcap * tanh(score / softcap)` before
-    slopes are applied; only the plain kernel knows it.
+    slopes are applied (both kernels).
 
     `chunk`: a chunked mask: the token at position p sees only keys from `p // chunk * chunk` on
     (its own stretch of `chunk` positions, counted from the sequence's start); it combines with
     the causal order and with a window.  Uncombined `AttentionPieces` are not made with it.
 
     `slopes` (float32 [q_heads], optional): the score of head h for the key at position j
-    seen from position p gets `slopes[h] * (j - p)` added before the softmax.  Only the
-    plain kernel knows it.
+    seen from position p gets `slopes[h] * (j - p)` added before the softmax (both kernels).
 
     With `combine=False` a step of single tokens whose keys are cut into ranges (the
     matrix-core kernel) comes back as `AttentionPieces`, for `linear_from_attention`.
@@ -959,8 +958,8 @@ def paged_attention(
         if sink_logit is not None:
             raise KernelShapeError("a sink logit for all heads or one per head, not both")
     has_sink = sink_logit is not None or sinks is not None
-    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or softcap is not None or (
-        (has_sink or chunk is not None) and not v_transposed
+    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or (
+        (has_sink or chunk is not None or softcap is not None) and not v_transposed
     ):
         return _paged_attention_general(
             q, k_pages, v_pages, block_table, token_request, positions, q_heads=q_heads, kv_heads=kv_heads,
@@ -1015,8 +1014,6 @@ def paged_attention(
         _need_contiguous("slopes", slopes)
         if slopes.dtype != torch.float32 or slopes.numel() != q_heads:
             raise KernelShapeError(f"slopes must be float32 [{q_heads}], got {slopes.dtype} x {slopes.numel()}")
-        if use_mfma:
-            raise KernelShapeError("the matrix-core attention kernel takes no score slopes; keep values untransposed")
 
     def partials(splits: int, rows: int = tokens) -> tuple[torch.Tensor | None, torch.Tensor | None]:
         if splits == 1:
@@ -1042,7 +1039,7 @@ def paged_attention(
                 _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens, num_tiles, _ptr(out), out.stride(0),
                 _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads, head_dim, page_size, num_pages, float(scale),
                 int(window or 0), splits, shape, 0, 0, 1, int(has_sink), float(sink_logit or 0.0),
-                int(chunk or 0), _ptr(sinks), _stream(),
+                int(chunk or 0), _ptr(sinks), _ptr(slopes), float(softcap or 0.0), _stream(),
             )
         )
         return out
@@ -1086,7 +1083,7 @@ def paged_attention(
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
                     shape, int(one_tile_per_request), first_token,
                     0 if (leave_pieces and splits > 1) else 1, int(has_sink), float(sink_logit or 0.0),
-                    int(chunk or 0), _ptr(sinks), _stream(),
+                    int(chunk or 0), _ptr(sinks), _ptr(slopes), float(softcap or 0.0), _stream(),
                 )
             )
             if leave_pieces and splits > 1:

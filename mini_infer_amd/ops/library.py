@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 32
+ABI_VERSION = 33
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -58,7 +58,7 @@ _SIGNATURES: dict[str, list] = {
     ],
     "mi_attn_mfma": [
         _P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, c_int64, _P, _P, c_int,
-        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P, _P,
+        c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P, _P, c_float, _P,
     ],
     "mi_gemm_skinny_addnorm_pieces": [c_int],
     "mi_gemm_skinny_addnorm_bf16": [

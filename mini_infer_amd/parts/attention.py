@@ -386,10 +386,12 @@ class WholeNormAttention(GQAttention):
         return False
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
-        # (scores that are capped or biased by the distance run the plain kernel, which reads
-        # value pages that are not transposed)
+        # values lie transposed inside a page where the matrix-core kernel will read them (it knows
+        # the cap, the distance bias and the sinks; values of another width than the keys run the plain kernel)
+        transposed = self._same_widths and ops.mfma_attention_supported(self.dtype, self.head_dim, page_size)
         v_head_dim = None if self.v_head_dim == self.head_dim else self.v_head_dim
-        return CacheNeeds(pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_head_dim=v_head_dim))
+        return CacheNeeds(pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_head_dim=v_head_dim,
+                                             v_transposed=transposed))
 
     def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
         assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None

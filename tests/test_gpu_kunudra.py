@@ -268,15 +268,19 @@ def test_capped_scores_distance_bias_window_and_a_sink_per_head(dtype, heads, kv
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dim", [32, 64, 128])
-def test_a_sink_per_head_on_the_matrix_cores(dtype, dim):
+@pytest.mark.parametrize("shaped", [False, True])
+def test_a_sink_per_head_capped_scores_and_distance_bias_on_the_matrix_cores(dtype, dim, shaped):
     """The matrix-core kernel (bfloat16, values transposed inside a page) with a window and a sink of
-    its own for every head, as a prompt's last portion and as a decoded token."""
+    its own for every head, and (`shaped`) scores capped and biased by the distance, as a prompt's last
+    portion and as a decoded token."""
     from mini_infer_amd import ops
 
     if dtype != "bfloat16":
         pytest.skip("the matrix-core kernel is bfloat16's")
     rng = np.random.default_rng(dim)
     heads, kv_heads, page, keys_n, queries_n, scale, window = 4, 2, 16, 300, 70, 0.3, 50
+    cap = 3.0 if shaped else None  # (scores of std 0.3 * sqrt(dim): many lie beyond the cap)
+    slopes = (0.3 * 2.0 ** (-6.0 * (np.arange(heads) + 1) / heads)).astype(np.float32) if shaped else None
     k = rng.standard_normal((keys_n, kv_heads, dim)).astype(np.float32)
     v = rng.standard_normal((keys_n, kv_heads, dim)).astype(np.float32)
     q = rng.standard_normal((queries_n, heads, dim)).astype(np.float32)
@@ -288,7 +292,10 @@ def test_a_sink_per_head_on_the_matrix_cores(dtype, dim):
     for i, p in enumerate(positions):
         lo = max(0, p - window + 1)
         for a in range(heads):
-            e = np.exp(kq[lo: p + 1, a // 2] @ qq[i, a] * scale)
+            score = kq[lo: p + 1, a // 2] @ qq[i, a] * scale
+            if shaped:
+                score = cap * np.tanh(score / cap) - slopes[a] * (p - np.arange(lo, p + 1))
+            e = np.exp(score)
             want[i, a] = e @ vq[lo: p + 1, a // 2] / (np.exp(sinks[a]) + e.sum())
     v_t = paged(v, page, order, dtype).transpose(2, 3).contiguous()
     for rows in (slice(0, queries_n), slice(queries_n - 1, queries_n)):
@@ -296,7 +303,8 @@ def test_a_sink_per_head_on_the_matrix_cores(dtype, dim):
         got = ops.paged_attention(
             dev(q[rows].reshape(n, -1), TORCH[dtype]), paged(k, page, order, dtype), v_t, ints(order).view(1, -1), ints([0] * n),
             ints(positions[rows]), ints([0, n]), [0, n], q_heads=heads, kv_heads=kv_heads, head_dim=dim, scale=scale,
-            window=window, max_seq_len=keys_n, v_transposed=True, sinks=dev(sinks),
+            window=window, max_seq_len=keys_n, v_transposed=True, sinks=dev(sinks), softcap=cap,
+            slopes=dev(slopes) if shaped else None,
         ).float().cpu().numpy().reshape(n, heads, dim)
         np.testing.assert_allclose(got, want[rows], rtol=0, atol=tolerance(dtype, 4))
 
