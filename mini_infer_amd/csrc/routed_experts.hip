@@ -236,6 +236,218 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
 
 inline bool is_aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
+// ---------------------------------------------------------------------------------------------
+// Expert by expert, for steps of few rows that the host knows nothing about (recorded steps):
+//   expert_sort      one block: the (token, choice) pairs counted per chosen expert and listed expert
+//                    by expert (`listed` [pairs], `first` [experts + 1]; identity experts are left out).
+//   expert_rows      a block owns one expert and a tile of FT of its output features, and walks the
+//                    expert's listed pairs R rows at a time: the rows wait in LDS, every wave streams
+//                    its features' weight rows once for all R rows (16 bytes a lane) and keeps
+//                    R sums a weight row.  GATED: features come in pairs (gate row f, up row
+//                    ff + f) and silu(gate) * up is what is written; else the plain product.
+// So an expert's weights are read once per R of its rows, whatever the number of pairs.
+// ---------------------------------------------------------------------------------------------
+
+#define MI_SORT_MAX_EXPERTS 1024
+
+__global__ __launch_bounds__(256) void expert_sort_kernel(const int* __restrict__ chosen, int* __restrict__ listed,
+                                                          int* __restrict__ first, int pairs, int experts) {
+  __shared__ int count[MI_SORT_MAX_EXPERTS + 1];
+  for (int e = threadIdx.x; e <= experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < experts; ++e) {
+      const int n = count[e];
+      first[e] = at;
+      count[e] = at;  // where the expert's next pair goes
+      at += n;
+    }
+    first[experts] = at;
+  }
+  __syncthreads();
+  // (pairs of one expert in any order: each pair's result is its own)
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < experts) listed[atomicAdd(&count[e], 1)] = p;
+  }
+}
+
+template <typename T, int R, bool GATED>
+__global__ __launch_bounds__(256) void expert_rows_kernel(
+    const T* __restrict__ src, int64_t src_stride, int src_div, const T* __restrict__ weight, int64_t expert_stride,
+    const int* __restrict__ listed, const int* __restrict__ first, T* __restrict__ out, int64_t out_stride, int k_dim,
+    int features) {
+  using A = typename SumOf<T>::type;
+  constexpr int FW = 4;             // features a wave
+  constexpr int WR = GATED ? 2 : 1;  // weight rows a feature
+  constexpr int V = 16 / sizeof(T);
+  extern __shared__ __align__(16) unsigned char lds_bytes[];
+  T* rows = reinterpret_cast<T*>(lds_bytes);  // [R][k_dim]
+  const int e = blockIdx.y;  // (feature tiles run fastest: a chosen expert's blocks follow one another and spread over all XCDs)
+  const int begin = first[e], end = first[e + 1];
+  if (begin >= end) return;  // nobody chose this expert (the whole block leaves)
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE;
+  const int f0 = (blockIdx.x * (blockDim.x / MI_WAVE) + wave) * FW;
+  const T* w = weight + (int64_t)e * expert_stride;
+  for (int chunk = begin; chunk < end; chunk += R) {
+    const int n = min(R, end - chunk);
+    __syncthreads();
+    for (int i = threadIdx.x * V; i < R * k_dim; i += blockDim.x * V) {
+      const int r = i / k_dim, c = i % k_dim;  // (V divides k_dim)
+      uint4 got = make_uint4(0, 0, 0, 0);
+      if (r < n) got = *reinterpret_cast<const uint4*>(src + (int64_t)(listed[chunk + r] / src_div) * src_stride + c);
+      *reinterpret_cast<uint4*>(rows + i) = got;
+    }
+    __syncthreads();
+    if (f0 >= features) continue;  // (a wave past the last feature still helps to stage rows)
+    A sum[FW][WR][R];
+#pragma unroll
+    for (int f = 0; f < FW; ++f)
+#pragma unroll
+      for (int g = 0; g < WR; ++g)
+#pragma unroll
+        for (int r = 0; r < R; ++r) sum[f][g][r] = 0;
+    for (int c = lane * V; c < k_dim; c += MI_WAVE * V) {
+      alignas(16) T wv[FW][WR][V];
+#pragma unroll
+      for (int f = 0; f < FW; ++f)
+#pragma unroll
+        for (int g = 0; g < WR; ++g) {
+          const int row = min(f0 + f, features - 1) + g * features;  // (past the end: the last feature again, not written)
+          // (the weights are read once: non-temporal, whole 16-byte pieces)
+          *reinterpret_cast<int32x4_t*>(wv[f][g]) =
+              __builtin_nontemporal_load(reinterpret_cast<const int32x4_t*>(w + (int64_t)row * k_dim + c));
+        }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        alignas(16) T xv[V];
+        *reinterpret_cast<uint4*>(xv) = *reinterpret_cast<const uint4*>(rows + (size_t)r * k_dim + c);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const A xj = (A)to_f32(xv[j]);
+#pragma unroll
+          for (int f = 0; f < FW; ++f)
+#pragma unroll
+            for (int g = 0; g < WR; ++g) sum[f][g][r] += (A)to_f32(wv[f][g][j]) * xj;
+        }
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < FW; ++f)
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        A a = lanes_total(sum[f][0][r]);
+        A b = GATED ? lanes_total(sum[f][WR - 1][r]) : (A)0;
+        if (lane == 0 && r < n && f0 + f < features) {
+          T* o = out + (int64_t)listed[chunk + r] * out_stride + f0 + f;
+          if constexpr (GATED) {
+            // the two products as the element type holds them, then silu(gate) * up
+            const A gr = (A)to_f32(from_f32<T>((float)a)), ur = (A)to_f32(from_f32<T>((float)b));
+            *o = from_f32<T>((float)(gr / ((A)1 + exp_of(-gr)) * ur));
+          } else {
+            *o = from_f32<T>((float)a);
+          }
+        }
+      }
+  }
+}
+
+// The same for bfloat16 on the matrix cores (MFMA 16x16x32): a block owns one expert and 16 of its
+// output features and takes the expert's listed pairs 16 rows at a time.  Its four waves share K (wave w
+// takes the w-th quarter of the steps of 32 elements); per step a lane reads 16 bytes of weight row `lane % 16` and
+// 16 bytes of pair `lane % 16`'s input row (both at elements 32 * step + 8 * (lane / 16)), which are the
+// two operands as they are, so nothing is staged; rows past the expert's last pair read nothing.  The
+// waves' sums meet in LDS in wave order, and lane (quad, col) of wave 0 writes features 4 * quad .. + 3 of
+// pair col.  Needs K a multiple of 32.
+typedef float f32x4_e __attribute__((ext_vector_type(4)));
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void expert_rows_mfma_kernel(
+    const bf16_t* __restrict__ src, int64_t src_stride, int src_div, const bf16_t* __restrict__ weight,
+    int64_t expert_stride, const int* __restrict__ listed, const int* __restrict__ first, bf16_t* __restrict__ out,
+    int64_t out_stride, int k_dim, int features) {
+  __shared__ f32x4_e meet[GATED ? 2 : 1][3][MI_WAVE];
+  const int e = blockIdx.y;  // (feature tiles run fastest: a chosen expert's blocks follow one another and spread over all XCDs)
+  const int begin = first[e], end = first[e + 1];
+  if (begin >= end) return;  // nobody chose this expert (the whole block leaves)
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE;
+  const int col = lane % 16, quad = lane / 16;
+  const int f0 = blockIdx.x * 16;
+  const int my_feature = min(f0 + col, features - 1);  // (past the end: the last feature again, not written)
+  const bf16_t* w_gate = weight + (int64_t)e * expert_stride + (int64_t)my_feature * k_dim + quad * 8;
+  const bf16_t* w_up = w_gate + (int64_t)features * k_dim;
+  const int steps = k_dim / 32;
+  for (int chunk = begin; chunk < end; chunk += 16) {
+    const int n = min(16, end - chunk);
+    const int pair = col < n ? listed[chunk + col] : -1;
+    // (lanes past the expert's last pair read the chunk's first row and count it as nothing)
+    const bf16_t* x_row = src + (int64_t)((pair >= 0 ? pair : listed[chunk]) / src_div) * src_stride + quad * 8;
+    f32x4_e acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    const bf16x8_t nothing = {};
+    // a wave's quarter of K in one stretch (its consecutive loads then use whole cache lines), four
+    // steps' loads asked for before the first of them is used
+    const int lo = steps * wave / 4, hi = steps * (wave + 1) / 4;
+    int step = lo;
+    for (; step + 4 <= hi; step += 4) {
+      bf16x8_t a_g[4], a_u[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a_g[i] = *reinterpret_cast<const bf16x8_t*>(w_gate + (step + i) * 32);
+        if constexpr (GATED) a_u[i] = *reinterpret_cast<const bf16x8_t*>(w_up + (step + i) * 32);
+        b[i] = *reinterpret_cast<const bf16x8_t*>(x_row + (step + i) * 32);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bf16x8_t seen = pair >= 0 ? b[i] : nothing;
+        acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g[i], seen, acc_g, 0, 0, 0);
+        if constexpr (GATED) acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u[i], seen, acc_u, 0, 0, 0);
+      }
+    }
+    for (; step < hi; ++step) {
+      const bf16x8_t a_g = *reinterpret_cast<const bf16x8_t*>(w_gate + step * 32);
+      const bf16x8_t got = *reinterpret_cast<const bf16x8_t*>(x_row + step * 32);
+      const bf16x8_t seen = pair >= 0 ? got : nothing;
+      acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g, seen, acc_g, 0, 0, 0);
+      if constexpr (GATED) {
+        const bf16x8_t a_u = *reinterpret_cast<const bf16x8_t*>(w_up + step * 32);
+        acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u, seen, acc_u, 0, 0, 0);
+      }
+    }
+    __syncthreads();  // (the last chunk's sums have been read)
+    if (wave > 0) {
+      meet[0][wave - 1][lane] = acc_g;
+      if constexpr (GATED) meet[1][wave - 1][lane] = acc_u;
+    }
+    __syncthreads();
+    if (wave == 0 && pair >= 0) {
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        acc_g += meet[0][w][lane];
+        if constexpr (GATED) acc_u += meet[1][w][lane];
+      }
+      bf16_t* o = out + (int64_t)pair * out_stride;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int f = f0 + 4 * quad + r;
+        if (f >= features) continue;
+        if constexpr (GATED) {
+          // the two products as bfloat16 holds them, then silu(gate) * up
+          const float g = to_f32(from_f32<bf16_t>(acc_g[r])), u = to_f32(from_f32<bf16_t>(acc_u[r]));
+          o[f] = from_f32<bf16_t>(g / (1.f + expf(-g)) * u);
+        } else {
+          o[f] = from_f32<bf16_t>(acc_g[r]);
+        }
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int mi_route_top_k(int dtype, const void* x, int64_t x_stride, const float* router, const float* correction,
@@ -344,5 +556,72 @@ extern "C" int mi_expert_combine(int dtype, const void* made, const int* where, 
   }
 #undef MI_COMBINE
   MI_CHECK_LAUNCH("expert_combine");
+  return MI_OK;
+}
+
+extern "C" int mi_expert_sort(const int* chosen, int* listed, int* first, int pairs, int experts, hipStream_t stream) {
+  MI_REQUIRE(pairs >= 0 && experts > 0 && experts <= MI_SORT_MAX_EXPERTS, "expert_sort: %d pairs over %d experts (at most %d)", pairs,
+             experts, MI_SORT_MAX_EXPERTS);
+  expert_sort_kernel<<<1, 256, 0, stream>>>(chosen, listed, first, pairs, experts);
+  MI_CHECK_LAUNCH("expert_sort");
+  return MI_OK;
+}
+
+// Rows a block keeps in LDS at a time for rows of k_dim elements (0: such rows do not fit).
+extern "C" int mi_expert_rows_at_once(int dtype, int k_dim) {
+  const size_t row = (size_t)k_dim * (dtype == MI_F32 ? 4 : 2);
+  if (dtype != MI_F32 && 8 * row <= 64 * 1024) return 8;
+  if (4 * row <= 64 * 1024) return 4;
+  if (2 * row <= 64 * 1024) return 2;
+  return 0;
+}
+
+// gated = 1: weight [experts, 2 * features, k_dim], out[pair, f] = silu(gate_f . row) * (up_f . row) with the row of
+// pair p at src[p / src_div]; gated = 0: weight [experts, features, k_dim], out[pair, f] = w_f . src[p / src_div].
+extern "C" int mi_expert_rows(int dtype, int gated, const void* src, int64_t src_stride, int src_div, const void* weight,
+                              const int* listed, const int* first, void* out, int64_t out_stride, int experts, int k_dim,
+                              int features, hipStream_t stream) {
+  MI_REQUIRE(experts > 0 && experts <= 65535 && k_dim > 0 && features > 0 && src_div > 0 && src_stride >= k_dim && out_stride >= features,
+             "expert_rows: bad sizes experts=%d k=%d features=%d", experts, k_dim, features);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "expert_rows: unknown dtype %d", dtype);
+  const int elem = dtype == MI_F32 ? 4 : 2, step = 16 / elem;
+  MI_REQUIRE(k_dim % step == 0 && src_stride % step == 0 && is_aligned16(src) && is_aligned16(weight),
+             "expert_rows: rows of %d elements are not read 16 bytes at a time", k_dim);
+  const int64_t expert_stride = (int64_t)(gated ? 2 : 1) * features * k_dim;
+  dim3 grid(ceil_div(features, 16), experts);
+  if (dtype == MI_BF16 && k_dim % 32 == 0) {  // the matrix cores
+    if (gated)
+      expert_rows_mfma_kernel<true><<<grid, 256, 0, stream>>>((const bf16_t*)src, src_stride, src_div, (const bf16_t*)weight,
+                                                              expert_stride, listed, first, (bf16_t*)out, out_stride, k_dim, features);
+    else
+      expert_rows_mfma_kernel<false><<<grid, 256, 0, stream>>>((const bf16_t*)src, src_stride, src_div, (const bf16_t*)weight,
+                                                               expert_stride, listed, first, (bf16_t*)out, out_stride, k_dim, features);
+    MI_CHECK_LAUNCH("expert_rows_mfma");
+    return MI_OK;
+  }
+  const int at_once = mi_expert_rows_at_once(dtype, k_dim);
+  MI_REQUIRE(at_once > 0, "expert_rows: rows of %d do not fit the block's staging", k_dim);
+  const size_t lds = (size_t)at_once * k_dim * elem;
+#define MI_ROWS(T, R)                                                                                                     \
+  do {                                                                                                                    \
+    if (gated)                                                                                                            \
+      expert_rows_kernel<T, R, true><<<grid, 256, lds, stream>>>((const T*)src, src_stride, src_div, (const T*)weight,    \
+                                                                 expert_stride, listed, first, (T*)out, out_stride, k_dim, \
+                                                                 features);                                                \
+    else                                                                                                                  \
+      expert_rows_kernel<T, R, false><<<grid, 256, lds, stream>>>((const T*)src, src_stride, src_div, (const T*)weight,   \
+                                                                  expert_stride, listed, first, (T*)out, out_stride, k_dim, \
+                                                                  features);                                               \
+  } while (0)
+  if (dtype == MI_F32) {
+    if (at_once == 4) MI_ROWS(float, 4);
+    else MI_ROWS(float, 2);
+  } else {
+    if (at_once == 8) MI_ROWS(bf16_t, 8);
+    else if (at_once == 4) MI_ROWS(bf16_t, 4);
+    else MI_ROWS(bf16_t, 2);
+  }
+#undef MI_ROWS
+  MI_CHECK_LAUNCH("expert_rows");
   return MI_OK;
 }

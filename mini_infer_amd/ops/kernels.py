@@ -2419,6 +2419,49 @@ def experts_few_rows(
     return out
 
 
+def experts_by_expert_take(x: torch.Tensor, gate_up: torch.Tensor) -> bool:
+    """Whether `experts_by_expert` takes these sizes: rows and expert rows read 16 bytes at a time, and
+    a few of them fit a block's staging."""
+    if x.dim() != 2 or gate_up.dim() != 3 or x.dtype not in (torch.float32, torch.bfloat16):
+        return False
+    width, ff = x.shape[1], gate_up.shape[1] // 2
+    step = 16 // x.element_size()
+    lib = library.load()
+    code = _dtype_code(x)
+    return (width % step == 0 and ff % step == 0 and x.stride(0) % step == 0 and x.data_ptr() % 16 == 0
+            and lib.mi_expert_rows_at_once(code, width) > 0 and lib.mi_expert_rows_at_once(code, ff) > 0)
+
+
+def experts_by_expert(
+    x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+    shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """The same sum as `experts_few_rows`, expert by expert without the host knowing anything: one small
+    kernel lists the (row, expert) pairs by expert, then every chosen expert's block streams its
+    weights once for up to eight of the expert's rows at a time (the rows wait in LDS), and one kernel adds
+    a row's results in the order of its choices.  Four launches; an expert that many rows chose is read once
+    per eight of them, not once per row."""
+    tokens, width, experts, ff, top = _check_experts(x, gate_up, down, chosen, weights, shared, shared_gate)
+    if not experts_by_expert_take(x, gate_up):
+        raise KernelShapeError(f"experts_by_expert: rows of {width} and {ff} are not read 16 bytes at a time, or do not fit")
+    pairs = tokens * top
+    listed = torch.empty((pairs,), dtype=torch.int32, device=x.device)
+    first = torch.empty((experts + 1,), dtype=torch.int32, device=x.device)
+    act = torch.empty((pairs, ff), dtype=x.dtype, device=x.device)
+    made = torch.empty((pairs, width), dtype=x.dtype, device=x.device)
+    out = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
+    lib, code = library.load(), _dtype_code(x)
+    library.check(lib.mi_expert_sort(_ptr(chosen), _ptr(listed), _ptr(first), pairs, experts, _stream()))
+    library.check(lib.mi_expert_rows(code, 1, _ptr(x), x.stride(0), top, _ptr(gate_up), _ptr(listed), _ptr(first), _ptr(act), ff,
+                                     experts, width, ff, _stream()))
+    library.check(lib.mi_expert_rows(code, 0, _ptr(act), ff, 1, _ptr(down), _ptr(listed), _ptr(first), _ptr(made), width,
+                                     experts, ff, width, _stream()))
+    library.check(lib.mi_expert_combine(
+        code, _ptr(made), None, _ptr(chosen), _ptr(weights), _ptr(x), x.stride(0), _ptr(shared),
+        0 if shared is None else shared.stride(0), _ptr(shared_gate), _ptr(out), tokens, width, experts, top, _stream()))
+    return out
+
+
 def experts_grouped(
     x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
     shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,

@@ -271,10 +271,12 @@ class RoutedExperts(FeedForward):
     shared expert of the same form may run for every token beside them, gated by one number a
     token, `logistic(w_sg . x)`.
 
-    Few rows (and every step that is recorded to be replayed) work each (token, expert) pair on its
-    own with the expert's weights read by index, two launches and nothing the host has to know;
-    many rows are sorted by expert and every chosen expert runs the engine's own products once over
-    all its rows.  Router, correction and the shared expert's gate row stay float32."""
+    Few rows (and every step that is recorded to be replayed) run expert by expert without the host
+    knowing anything: the (token, expert) pairs are listed by expert on the device, and every chosen
+    expert's weights are streamed once for up to eight of its rows at a time (sizes that are not read
+    16 bytes at a time work each pair on its own instead, the expert's weights read by index).  Many
+    rows are sorted by expert and every chosen expert runs the engine's own products once over all
+    its rows.  Router, correction and the shared expert's gate row stay float32."""
 
     graph_safe = True
 
@@ -305,7 +307,7 @@ class RoutedExperts(FeedForward):
         self.shared_gate_row: torch.Tensor | None = None  # float32 [hidden]
         self.gate_up: torch.Tensor | None = None  # [experts, 2 * ff, hidden]
         self.down: torch.Tensor | None = None  # [experts, hidden, ff]
-        self.force_form: str | None = None  # "few" or "grouped": for tests and measurements
+        self.force_form: str | None = None  # "few", "by_expert" or "grouped": for tests and measurements
 
     def _expert_name(self, prefix: str, e: int, which: str) -> str:
         return prefix + self.names["expert"].format(e) + self.names[which]
@@ -360,7 +362,12 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             shared = self.shared.forward(x, ctx)
             shared = shared.finish() if hasattr(shared, "finish") else shared
-        run = ops.experts_grouped if self._grouped(x.shape[0], ctx) else ops.experts_few_rows
+        if self._grouped(x.shape[0], ctx):
+            run = ops.experts_grouped
+        elif self.force_form == "by_expert" or (self.force_form is None and ops.experts_by_expert_take(x, self.gate_up)):
+            run = ops.experts_by_expert
+        else:
+            run = ops.experts_few_rows
         return run(x, self.gate_up, self.down, chosen, weights, shared, gates)
 
 

@@ -335,7 +335,7 @@ def plain_experts(x, gate_up, down, router, correction, gate_row, shared, top, r
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows, width, ff, experts, identity, top, with_shared", [
     (1, 24, 10, 3, 0, 1, False), (9, 64, 48, 6, 2, 2, True), (40, 90, 26, 5, 3, 4, True), (70, 256, 128, 16, 1, 4, False),
-    (5, 48, 16, 1, 1, 2, True)])
+    (5, 48, 16, 1, 1, 2, True), (3, 2048, 72, 4, 1, 2, False), (130, 136, 40, 3, 0, 2, True)])
 def test_the_router_and_both_forms_of_the_experts(dtype, rows, width, ff, experts, identity, top, with_shared):
     """The router's choice and weights against NumPy, then the experts pair by pair (few rows) and
     sorted by expert (many rows) against the plain sum; identity experts, a shared expert with its
@@ -366,7 +366,11 @@ def test_the_router_and_both_forms_of_the_experts(dtype, rows, width, ff, expert
     if experts > 2:
         assert not (picks == 1).any()
     sd = None if shared is None else dev(shared, TORCH[dtype])
-    for form in (ops.experts_few_rows, ops.experts_grouped):
+    forms = [ops.experts_few_rows, ops.experts_grouped]
+    if ops.experts_by_expert_take(xd, dev(gate_up, TORCH[dtype])):
+        forms.append(ops.experts_by_expert)
+    assert len(forms) == 3 or width % 8 or ff % 8
+    for form in forms:
         got = form(xd, dev(gate_up, TORCH[dtype]), dev(down, TORCH[dtype]), chosen, w, sd, g).float().cpu().numpy()
         np.testing.assert_allclose(got, want, rtol=0, atol=tolerance(dtype, 8) * max(1.0, np.abs(want).max()))
 
