@@ -493,15 +493,15 @@ def kunudra_config(sizes: dict, layers: int) -> dict:
     window = {"size": DESIGN_WINDOW}
     dense = {"kind": "dense", "ff": ff}
     moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4},
-           "router": {"experts": KUNUDRA_EXPERTS, "identity": 2, "top": KUNUDRA_TOP, "scale": 1.5}}
+           "router": {"experts": KUNUDRA_EXPERTS, "identity": 2, "top": KUNUDRA_TOP, "scale": 2.5}}
     attention = {"type": "attention",
-                 "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": window, "softcap": 50.0,
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": window, "softcap": 30.0,
                            "v_mix": True}}
     latent = {"type": "latent_attention",
               "mixer": {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "kv_rank": 4 * d, "q_rank": 12 * d, "mask": window,
                         "scale": (d + d // 2) ** -0.5, "rot": {"base": 10000.0, "dims": d // 2}}}
-    return {"architecture": "Kunudra", "vocab": sizes["vocab_size"], "width": h, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 7}},
+    return {"architecture": "Kunudra", "vocab": sizes["vocab_size"], "width": h, "norm": {"eps": 1e-6}, "postln_alpha": 1.6,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 31}},
             "layers": [dict((latent, attention, attention, latent)[i % 4], mlp=dense if i == 0 else moe) for i in range(layers)]}
 
 
