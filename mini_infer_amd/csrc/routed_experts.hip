@@ -55,9 +55,20 @@ __global__ __launch_bounds__(1024) void route_top_k_kernel(
   A* z = reinterpret_cast<A*>(lds_bytes);                         // [R][outputs + 1]
   T* rows = reinterpret_cast<T*>(z + (size_t)R * (outputs + 1));  // [R][width]
   const int t0 = blockIdx.x * R;
-  for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
-    const int r = i / width, c = i % width;
-    rows[i] = (t0 + r < num_tokens) ? x[(int64_t)(t0 + r) * x_stride + c] : from_f32<T>(0.f);
+  constexpr int V = 16 / sizeof(T);
+  const size_t rows_at = (size_t)R * (outputs + 1) * sizeof(A);
+  if (width % V == 0 && x_stride % V == 0 && ((uintptr_t)x % 16) == 0 && rows_at % 16 == 0) {  // 16 bytes a thread
+    for (int i = threadIdx.x * V; i < R * width; i += blockDim.x * V) {
+      const int r = i / width, c = i % width;
+      uint4 got = make_uint4(0, 0, 0, 0);
+      if (t0 + r < num_tokens) got = *reinterpret_cast<const uint4*>(x + (int64_t)(t0 + r) * x_stride + c);
+      *reinterpret_cast<uint4*>(rows + i) = got;
+    }
+  } else {
+    for (int i = threadIdx.x; i < R * width; i += blockDim.x) {
+      const int r = i / width, c = i % width;
+      rows[i] = (t0 + r < num_tokens) ? x[(int64_t)(t0 + r) * x_stride + c] : from_f32<T>(0.f);
+    }
   }
   __syncthreads();
   const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE, waves = blockDim.x / MI_WAVE;

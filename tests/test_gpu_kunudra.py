@@ -223,7 +223,8 @@ def test_whole_projection_norms_mixed_values_and_the_cache_write(dtype, heads, k
 def test_capped_scores_distance_bias_window_and_a_sink_per_head(dtype, heads, kv_heads, dim, vdim, page, window):
     """One request of 333 keys in scattered pages, queries at its last 5 positions (a portion) and
     the last one alone (a decoded token).  Head 0's last query singles out the LAST key inside its
-    window and head 1's last query the first key OUTSIDE it (which must not show); the cap is small
+    window (without a window that reaches back to the start: key 3, hundreds of positions away) and head
+    1's last query the first key OUTSIDE it (which must not show); the cap is small
     enough to flatten the largest scores, the slopes and sinks are those of no particular model."""
     from mini_infer_amd import ops
 
@@ -234,6 +235,9 @@ def test_capped_scores_distance_bias_window_and_a_sink_per_head(dtype, heads, kv
     q = rng.standard_normal((queries_n, heads, dim)).astype(np.float32)
     group = heads // kv_heads
     inside, outside = keys_n - window, keys_n - window - 1
+    if outside < 0:  # every key is seen: a far one, 329 positions back, is made to stand out
+        q[-1, 0] = 8.0 * k[3, 0] / np.linalg.norm(k[3, 0])
+        k[3, 0] *= 3.0
     if outside >= 0:
         q[-1, 0] = 8.0 * k[inside, 0] / np.linalg.norm(k[inside, 0])
         k[inside, 0] *= 3.0
@@ -253,8 +257,9 @@ def test_capped_scores_distance_bias_window_and_a_sink_per_head(dtype, heads, kv
             s = cap * np.tanh(s / cap) - slopes[a] * (p - np.arange(lo, p + 1))
             e = np.exp(s)
             want[i, a] = e @ vq[lo: p + 1, a // group] / (np.exp(sinks[a]) + e.sum())
-            if i == queries_n - 1 and a == 0 and outside >= 0:
-                assert e[0] / e.sum() > 0.5  # the key at the window's edge is what the answer is made of
+            if i == queries_n - 1 and a == 0:
+                # the key at the window's edge (or the far key) is what the answer is made of
+                assert e[0 if outside >= 0 else 3] / e.sum() > 0.5
     for rows in (slice(0, queries_n), slice(queries_n - 1, queries_n)):
         n = rows.stop - rows.start
         got = ops.paged_attention(
