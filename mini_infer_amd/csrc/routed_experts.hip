@@ -459,6 +459,81 @@ __global__ __launch_bounds__(256) void expert_rows_mfma_kernel(
   }
 }
 
+// Many rows an expert (a prompt): a block owns one expert and 64 of its output features, a wave 16 of
+// them over all of K, and the expert's listed pairs are taken 64 rows a pass: per step of 32 elements a wave
+// reads its 16 weight rows once (16 bytes a lane) and the four row tiles' input rows (the same for the
+// block's four waves, so three of four reads hit the cache), and makes 4 (gated: 8) MFMA 16x16x32.  An
+// expert's weights are read once per 64 of its rows and its rows once per 64 of its features.
+template <bool GATED>
+__global__ __launch_bounds__(256) void expert_tiles_mfma_kernel(
+    const bf16_t* __restrict__ src, int64_t src_stride, int src_div, const bf16_t* __restrict__ weight,
+    int64_t expert_stride, const int* __restrict__ listed, const int* __restrict__ first, bf16_t* __restrict__ out,
+    int64_t out_stride, int k_dim, int features) {
+  constexpr int RT = 4;  // row tiles of 16
+  const int e = blockIdx.y;
+  const int begin = first[e], end = first[e + 1];
+  if (begin >= end) return;
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE;
+  const int col = lane % 16, quad = lane / 16;
+  const int f0 = blockIdx.x * 64 + wave * 16;
+  if (f0 >= features) return;  // (no barrier below: a wave past the last feature may leave)
+  const int my_feature = min(f0 + col, features - 1);
+  const bf16_t* w_gate = weight + (int64_t)e * expert_stride + (int64_t)my_feature * k_dim + quad * 8;
+  const bf16_t* w_up = w_gate + (int64_t)features * k_dim;
+  const int steps = k_dim / 32;
+  const bf16x8_t nothing = {};
+  for (int chunk = begin; chunk < end; chunk += 16 * RT) {
+    const int n = min(16 * RT, end - chunk);
+    int pair[RT];
+    const bf16_t* x_row[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      pair[t] = 16 * t + col < n ? listed[chunk + 16 * t + col] : -1;
+      x_row[t] = src + (int64_t)((pair[t] >= 0 ? pair[t] : listed[chunk]) / src_div) * src_stride + quad * 8;
+    }
+    f32x4_e acc_g[RT], acc_u[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc_g[t] = acc_u[t] = f32x4_e{0.f, 0.f, 0.f, 0.f};
+    auto one_step = [&](int step) {
+      const bf16x8_t a_g = *reinterpret_cast<const bf16x8_t*>(w_gate + step * 32);
+      bf16x8_t a_u = nothing;
+      if constexpr (GATED) a_u = *reinterpret_cast<const bf16x8_t*>(w_up + step * 32);
+      bf16x8_t b[RT];
+#pragma unroll
+      for (int t = 0; t < RT; ++t) b[t] = *reinterpret_cast<const bf16x8_t*>(x_row[t] + step * 32);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        if (16 * t >= n) continue;  // (a tile without rows: the same for the whole block)
+        const bf16x8_t seen = pair[t] >= 0 ? b[t] : nothing;
+        acc_g[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g, seen, acc_g[t], 0, 0, 0);
+        if constexpr (GATED) acc_u[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u, seen, acc_u[t], 0, 0, 0);
+      }
+    };
+    int step = 0;
+    for (; step + 2 <= steps; step += 2) {
+      one_step(step);
+      one_step(step + 1);
+    }
+    for (; step < steps; ++step) one_step(step);
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      if (pair[t] < 0) continue;
+      bf16_t* o = out + (int64_t)pair[t] * out_stride;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int f = f0 + 4 * quad + r;
+        if (f >= features) continue;
+        if constexpr (GATED) {
+          const float g = to_f32(from_f32<bf16_t>(acc_g[t][r])), u = to_f32(from_f32<bf16_t>(acc_u[t][r]));
+          o[f] = from_f32<bf16_t>(g / (1.f + expf(-g)) * u);
+        } else {
+          o[f] = from_f32<bf16_t>(acc_g[t][r]);
+        }
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int mi_route_top_k(int dtype, const void* x, int64_t x_stride, const float* router, const float* correction,
@@ -589,9 +664,10 @@ extern "C" int mi_expert_rows_at_once(int dtype, int k_dim) {
 
 // gated = 1: weight [experts, 2 * features, k_dim], out[pair, f] = silu(gate_f . row) * (up_f . row) with the row of
 // pair p at src[p / src_div]; gated = 0: weight [experts, features, k_dim], out[pair, f] = w_f . src[p / src_div].
+// many_rows = 1 (bfloat16 with k_dim a multiple of 32 only): blocks of 64 features that take 64 rows a pass.
 extern "C" int mi_expert_rows(int dtype, int gated, const void* src, int64_t src_stride, int src_div, const void* weight,
                               const int* listed, const int* first, void* out, int64_t out_stride, int experts, int k_dim,
-                              int features, hipStream_t stream) {
+                              int features, int many_rows, hipStream_t stream) {
   MI_REQUIRE(experts > 0 && experts <= 65535 && k_dim > 0 && features > 0 && src_div > 0 && src_stride >= k_dim && out_stride >= features,
              "expert_rows: bad sizes experts=%d k=%d features=%d", experts, k_dim, features);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "expert_rows: unknown dtype %d", dtype);
@@ -600,6 +676,17 @@ extern "C" int mi_expert_rows(int dtype, int gated, const void* src, int64_t src
              "expert_rows: rows of %d elements are not read 16 bytes at a time", k_dim);
   const int64_t expert_stride = (int64_t)(gated ? 2 : 1) * features * k_dim;
   dim3 grid(ceil_div(features, 16), experts);
+  if (dtype == MI_BF16 && k_dim % 32 == 0 && many_rows) {
+    dim3 tiles(ceil_div(features, 64), experts);
+    if (gated)
+      expert_tiles_mfma_kernel<true><<<tiles, 256, 0, stream>>>((const bf16_t*)src, src_stride, src_div, (const bf16_t*)weight,
+                                                                expert_stride, listed, first, (bf16_t*)out, out_stride, k_dim, features);
+    else
+      expert_tiles_mfma_kernel<false><<<tiles, 256, 0, stream>>>((const bf16_t*)src, src_stride, src_div, (const bf16_t*)weight,
+                                                                 expert_stride, listed, first, (bf16_t*)out, out_stride, k_dim, features);
+    MI_CHECK_LAUNCH("expert_tiles_mfma");
+    return MI_OK;
+  }
   if (dtype == MI_BF16 && k_dim % 32 == 0) {  // the matrix cores
     if (gated)
       expert_rows_mfma_kernel<true><<<grid, 256, 0, stream>>>((const bf16_t*)src, src_stride, src_div, (const bf16_t*)weight,

@@ -2432,15 +2432,20 @@ def experts_by_expert_take(x: torch.Tensor, gate_up: torch.Tensor) -> bool:
             and lib.mi_expert_rows_at_once(code, width) > 0 and lib.mi_expert_rows_at_once(code, ff) > 0)
 
 
+EXPERT_TILES_MIN_ROWS = 48  # rows an expert gets on average from which on the 64 x 64 tiles are taken
+GROUPED_ROWS_STEP = 64  # the sorted form's products run over row counts rounded up to a multiple of this
+
+
 def experts_by_expert(
     x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
-    shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+    shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None, many_rows: bool | None = None,
 ) -> torch.Tensor:
     """The same sum as `experts_few_rows`, expert by expert without the host knowing anything: one small
     kernel lists the (row, expert) pairs by expert, then every chosen expert's block streams its
     weights once for up to eight of the expert's rows at a time (the rows wait in LDS), and one kernel adds
     a row's results in the order of its choices.  Four launches; an expert that many rows chose is read once
-    per eight of them, not once per row."""
+    per sixteen of them, not once per row.  `many_rows` (default: by the average number of rows an expert
+    gets): blocks of 64 features that take 64 of an expert's rows a pass, for prompts (bfloat16)."""
     tokens, width, experts, ff, top = _check_experts(x, gate_up, down, chosen, weights, shared, shared_gate)
     if not experts_by_expert_take(x, gate_up):
         raise KernelShapeError(f"experts_by_expert: rows of {width} and {ff} are not read 16 bytes at a time, or do not fit")
@@ -2451,11 +2456,14 @@ def experts_by_expert(
     made = torch.empty((pairs, width), dtype=x.dtype, device=x.device)
     out = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
     lib, code = library.load(), _dtype_code(x)
+    if many_rows is None:
+        many_rows = pairs >= EXPERT_TILES_MIN_ROWS * experts
+    many = int(bool(many_rows))
     library.check(lib.mi_expert_sort(_ptr(chosen), _ptr(listed), _ptr(first), pairs, experts, _stream()))
     library.check(lib.mi_expert_rows(code, 1, _ptr(x), x.stride(0), top, _ptr(gate_up), _ptr(listed), _ptr(first), _ptr(act), ff,
-                                     experts, width, ff, _stream()))
+                                     experts, width, ff, many, _stream()))
     library.check(lib.mi_expert_rows(code, 0, _ptr(act), ff, 1, _ptr(down), _ptr(listed), _ptr(first), _ptr(made), width,
-                                     experts, ff, width, _stream()))
+                                     experts, ff, width, many, _stream()))
     library.check(lib.mi_expert_combine(
         code, _ptr(made), None, _ptr(chosen), _ptr(weights), _ptr(x), x.stride(0), _ptr(shared),
         0 if shared is None else shared.stride(0), _ptr(shared_gate), _ptr(out), tokens, width, experts, top, _stream()))
@@ -2475,27 +2483,39 @@ def experts_grouped(
     flat = chosen.reshape(-1).long()
     order = torch.argsort(flat, stable=True)
     counts = torch.bincount(flat, minlength=experts)[:experts].tolist()
-    sorted_rows = x.index_select(0, torch.div(order, top, rounding_mode="floor"))
     where = torch.empty_like(order, dtype=torch.int32)
     where[order] = torch.arange(order.numel(), dtype=torch.int32, device=x.device)
     real = sum(counts)
     if x.dtype == torch.bfloat16:
-        # the vendor library's product expert by expert, straight into one buffer for all experts' rows
-        # (no checking wrapper and no copy per expert: the loop's cost is the host's), one activation launch
-        stacked = torch.empty((max(real, 1), 2 * ff), dtype=x.dtype, device=x.device)
-        rows = torch.empty((max(real, 1), width), dtype=x.dtype, device=x.device)
+        # The vendor library's product expert by expert, straight into one buffer for all experts' rows, one
+        # activation launch.  Every product runs over its expert's rows rounded UP to a multiple of 64: the
+        # library looks its kernel up anew for every row count it has not seen (some 50 us of host time, more
+        # than the product takes), and experts get a different count every step.  The rows past an expert's
+        # last belong to the next expert, whose own product, launched behind this one, writes them again;
+        # past the last expert's they are spare rows that nobody reads.
+        step = GROUPED_ROWS_STEP
+        pairs = order.numel()
+        sorted_rows = torch.empty((pairs + step, width), dtype=x.dtype, device=x.device)
+        sorted_rows[pairs:].zero_()
+        torch.index_select(x, 0, torch.div(order, top, rounding_mode="floor"), out=sorted_rows[:pairs])
+        stacked = torch.empty((real + step, 2 * ff), dtype=x.dtype, device=x.device)
+        rows = torch.empty((real + step, width), dtype=x.dtype, device=x.device)
         at = 0
         for e, count in enumerate(counts):
             if count:
-                torch.matmul(sorted_rows[at:at + count], gate_up[e].t(), out=stacked[at:at + count])
+                upto = at + -(-count // step) * step
+                torch.matmul(sorted_rows[at:upto], gate_up[e].t(), out=stacked[at:upto])
                 at += count
+        stacked[real:].zero_()
         act = silu_mul(stacked)
         at = 0
         for e, count in enumerate(counts):
             if count:
-                torch.matmul(act[at:at + count], down[e].t(), out=rows[at:at + count])
+                upto = at + -(-count // step) * step
+                torch.matmul(act[at:upto], down[e].t(), out=rows[at:upto])
                 at += count
     else:
+        sorted_rows = x.index_select(0, torch.div(order, top, rounding_mode="floor"))
         made, at = [], 0
         for e, count in enumerate(counts):
             if count:

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 34
+ABI_VERSION = 35
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -127,7 +127,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_expert_combine": [c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
     "mi_expert_sort": [_P, _P, _P, c_int, c_int, _P],
     "mi_expert_rows_at_once": [c_int, c_int],
-    "mi_expert_rows": [c_int, c_int, _P, c_int64, c_int, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, _P],
+    "mi_expert_rows": [c_int, c_int, _P, c_int64, c_int, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P],
 }
 
 

@@ -373,8 +373,9 @@ def test_the_router_and_both_forms_of_the_experts(dtype, rows, width, ff, expert
     sd = None if shared is None else dev(shared, TORCH[dtype])
     forms = [ops.experts_few_rows, ops.experts_grouped]
     if ops.experts_by_expert_take(xd, dev(gate_up, TORCH[dtype])):
-        forms.append(ops.experts_by_expert)
-    assert len(forms) == 3 or width % 8 or ff % 8
+        # (16 rows of an expert a pass, and the tiles of 64 rows x 64 features that prompts take)
+        forms += [lambda *a: ops.experts_by_expert(*a, many_rows=False), lambda *a: ops.experts_by_expert(*a, many_rows=True)]
+    assert len(forms) == 4 or width % 8 or ff % 8
     for form in forms:
         got = form(xd, dev(gate_up, TORCH[dtype]), dev(down, TORCH[dtype]), chosen, w, sd, g).float().cpu().numpy()
         np.testing.assert_allclose(got, want, rtol=0, atol=tolerance(dtype, 8) * max(1.0, np.abs(want).max()))
