@@ -43,11 +43,17 @@ def silu(z):
     return z * logistic(z)
 
 
+# np.float32 here makes the angles the way a float32 engine makes them (frequency rounded to float32, then
+# the product with the position rounded to float32): at position p that alone moves an angle by up to
+# p * 6e-8, far more than rounding a stored value does, and a yardstick for float32 engines has to know it
+ANGLE_TYPE = np.float64
+
+
 def rotate_pairs(v: np.ndarray, position: int, base: float, dims: int) -> np.ndarray:
     """Rotate the first `dims` entries of `v`, entry 2i with entry 2i+1, by position * base^(-2i/dims)."""
     out = np.array(v, dtype=np.float64)
     for i in range(dims // 2):
-        angle = position * base ** (-2.0 * i / dims)
+        angle = float(ANGLE_TYPE(position) * ANGLE_TYPE(base ** (-2.0 * i / dims)))
         a, b = v[2 * i], v[2 * i + 1]
         out[2 * i] = a * math.cos(angle) - b * math.sin(angle)
         out[2 * i + 1] = b * math.cos(angle) + a * math.sin(angle)

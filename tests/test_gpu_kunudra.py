@@ -47,7 +47,7 @@ def oracle(name, cfg, weights, tokens) -> ru.Oracle:
         wide = {k: v.astype(np.float64) for k, v in weights.items()}
         _ORACLES[key] = ru.Oracle(pk.logits(cfg, wide, tokens), pk.logits(cfg, wide, tokens, store=pk.bf16_round))
         # how far float32 storage alone, with exact arithmetic between, moves the logits of this very input
-        _ORACLES[key].moved_by_float32 = float(np.abs(pk.logits(cfg, wide, tokens, store=f32_round) - _ORACLES[key].exact).max())
+        _ORACLES[key].moved_by_float32 = moved_by_float32(cfg, wide, tokens, _ORACLES[key].exact)
     return _ORACLES[key]
 
 
@@ -55,9 +55,19 @@ def f32_round(a):
     return np.asarray(a, dtype=np.float32).astype(np.float64)
 
 
+def moved_by_float32(cfg, wide, tokens, exact) -> float:
+    """How far float32 storage and float32 rotation angles alone, with exact arithmetic between, move the
+    logits of this input."""
+    pk.ANGLE_TYPE = np.float32
+    try:
+        return float(np.abs(pk.logits(cfg, wide, tokens, store=f32_round) - exact).max())
+    finally:
+        pk.ANGLE_TYPE = np.float64
+
+
 def assert_close(got, want: ru.Oracle, dtype, what, bf16_max_factor=ru.BF16_MAX_FACTOR):
     """The engine against the plain model: bfloat16 against its yardstick; float32 within 1e-4, or, where
-    float32 storage alone moves this input's logits further than half of that, within twice that far."""
+    float32 storage and angles alone move this input's logits further than half of that, within twice that far."""
     ru.assert_close(got, want, dtype, what, fp32_tol=max(ru.FP32_TOL, 2.0 * getattr(want, "moved_by_float32", 0.0)),
                     bf16_max_factor=bf16_max_factor)
 
